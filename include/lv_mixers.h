@@ -25,6 +25,15 @@
  *   lv_relu2_scale           squared relu of the experts' up projections times the routing weight
  *   lv_moe_grouped_ff        the experts' feed-forward on rows sorted by expert (grouped GEMMs on the matrix cores)
  *   lv_moe_sort, lv_moe_combine   its first and last step alone, for callers that multiply the sorted rows themselves
+ *   lv_sandwich_add_norm     single f32 residual of layers that norm both sides of a sublayer: adds the RMS-normed
+ *                            sublayer output, a row of activations and a vector, RMS norm with weight (offset + w)
+ *   lv_rotary_store          rotation of part of every query and key head, a factor per query head, K/V scatter
+ *                            into the paged cache
+ *   lv_polynorm              c1 R(z) + c2 R(z^2) + c3 R(z^3) + c0 with R the division by a row's root mean square
+ *   lv_expert_glu            clamped gated unit of several experts side by side with a factor per (token, expert)
+ *                            on the pre-activations and a sigmoid per token on the result
+ *   lv_moe_grouped_glu_ff    the gathered feed-forward for clamped gated experts whose routing weight scales the
+ *                            expert's input
  *
  * A "ragged step" is a batch of B sequences; sequence b brings cu_q[b+1]-cu_q[b] new tokens that
  * follow ctx_lens[b] tokens already in the cache / state (a whole prompt, a portion of one, or one
@@ -46,7 +55,7 @@
 extern "C" {
 #endif
 
-#define LV_MIX_ABI_VERSION 5
+#define LV_MIX_ABI_VERSION 6
 #define LV_MIX_BF16 0
 #define LV_MIX_F32 1
 #define LV_MIX_MAX_STREAMS 8
@@ -119,14 +128,15 @@ int lv_pool_update(const void* k_cache, const void* v_cache, void* kp, void* vp,
 
 /* Query at position i sees cached positions j with 0 <= i-j < window and every pooled block b with
  * b*P + P - 1 <= i - window (P == 0: no pooled blocks); weights exp(s) / (sink + sum exp(s)) with
- * sink = 1 for has_sink, else 0.  gate (optional) act rows of stride ld_gate: out *= sigmoid(gate).
+ * sink = 1 for has_sink, else 0.  gate (optional) act rows of stride ld_gate holding H*Dv numbers
+ * (LV_MIX_GATE_PER_CHANNEL) or H (LV_MIX_GATE_PER_HEAD): out *= sigmoid(gate).
  * q act [T, H*D] contiguous; out act [T, H*Dv].  k_ld, v_ld: elements between two tokens' rows in k_cache and v_cache
  * (0: G*D and G*Dv); the pooled caches are always dense. */
 int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
                         const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                         const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G,
                         int D, int Dv, int page, int window, int P, float scale, int has_sink, int64_t k_ld,
-                        int64_t v_ld, int dtype, void* stream);
+                        int64_t v_ld, int gate_kind, int dtype, void* stream);
 
 /* The same attention on the matrix cores: bf16 only, D and Dv multiples of 16 up to 256. Tiles of 16 new
  * tokens per sequence; max_new_tokens = the largest cu_q[b+1] - cu_q[b] of the step.
@@ -136,7 +146,7 @@ int lv_window_pool_attn_mfma(const void* q, const void* k_cache, const void* v_c
                              const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                              const int32_t* block_tables, int bt_stride, int B, int max_new_tokens, int H, int G, int D,
                              int Dv, int page, int window, int P, float scale, int has_sink, int nsplit, void* workspace,
-                             int64_t T, int64_t k_ld, int64_t v_ld, void* stream);
+                             int64_t T, int64_t k_ld, int64_t v_ld, int gate_kind, void* stream);
 
 /* Latent attention, step 1. proj act [T, ld]: the query latent at column off_q (Rq wide), the key/value latent at
  * off_kv (R wide) directly followed by the positional key part (Dr wide, may be 0).
@@ -162,10 +172,11 @@ int lv_latent_out_gate(const void* o, const void* gate, int64_t ld_gate, int gat
 /* Router of a mixture of experts. logits f32 [T, E]; scores s = sigmoid(logits); selection scores c = s + correction
  * (f32 [E], may be NULL). The experts are split into `groups` consecutive blocks of equal size; a block is ranked by its
  * two highest selection scores added up (by its one, for blocks of one expert); experts outside the `keep` highest-ranked blocks are excluded
- * (groups <= 1: all). The `top` largest c are chosen (ties: lowest index first); weights = their s / (sum + 1e-20).
+ * (groups <= 1: all). The `top` largest c are chosen (ties: lowest index first); weights = their s / (sum + 1e-20),
+ * or their s as they are when `normalize` is 0.
  * ids int32 [T, top], weights f32 [T, top], dense f32 [T, E] (weights at the chosen experts, 0 elsewhere; may be NULL). */
 int lv_moe_route(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
-                 int top, int groups, int keep, void* stream);
+                 int top, int groups, int keep, int normalize, void* stream);
 
 /* up act [T, E*F] (all experts' up projections side by side), dense f32 [T, E]:
  * out act [T, E*F] = relu(up)^2 * dense[t, e]. */
@@ -186,9 +197,46 @@ int64_t lv_moe_grouped_workspace_bytes(int64_t T, int W, int F, int E, int top);
  * multiple of `align`, so an expert owns rows [offsets[e], offsets[e + 1]), the last ones of which may be padding that the
  * kernel does not write: sorted_pair has room for M + E * align entries and is cleared by the caller. */
 int lv_moe_sort(const void* ids, int64_t M, int E, int align, void* sorted_pair, void* inv, void* offsets, void* stream);
-/* rows bf16 [M, W] (expert outputs in sorted order), inv int32 [T, top], weights f32 [T, top]:
+/* rows bf16 [M, W] (expert outputs in sorted order), inv int32 [T, top], weights f32 [T, top] (NULL: all one):
  * out bf16 [T, W] = sum_k weights[t, k] * rows[inv[t, k]] in f32; W a multiple of 4. */
 int lv_moe_combine(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top, void* stream);
+
+
+/* x f32 [T, W] in place:  x += y / sqrt(mean(y^2) + eps) * (w_offset + post_w)   (y act [T, W] with post_w f32 [W]; both NULL: skipped)
+ *                         x += rows + vec                                         (rows act [T, W], vec f32 [W]; either may be NULL)
+ * out act [T, W] = x / sqrt(mean(x^2) + eps) * (w_offset + w)  (out and w may be NULL: update only). All arithmetic f32. */
+int lv_sandwich_add_norm(void* x, const void* y, const void* post_w, const void* rows, const void* vec, const void* w,
+                         float w_offset, void* out, int64_t T, int W, float eps, int dtype, void* stream);
+
+/* proj act [T, ld]: H query heads of D at column off_q, G key heads of D at off_k, G value heads of Dv at off_v.
+ * The first rot_dims (even, <= D) entries of every query and key head are rotated: entry i pairs with i + rot_dims/2,
+ * angle = position * inv_freq[i] (f32 [rot_dims/2]), position = ctx_lens[b] + index in the step; query head h is then
+ * multiplied by head_scale[h] (f32 [H], may be NULL).  q_out act [T, H*D] contiguous; rotated keys into
+ * k_cache [pages, page, G, D] and values into v_cache [pages, page, G, Dv] at the token's slot. */
+int lv_rotary_store(const void* proj, int64_t ld, int off_q, int off_k, int off_v, const void* inv_freq,
+                    const void* head_scale, void* q_out, void* k_cache, void* v_cache, const int32_t* cu_q,
+                    const int32_t* ctx_lens, const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T,
+                    int H, int G, int D, int Dv, int rot_dims, int page, int dtype, void* stream);
+
+/* in act [T, F] (row stride ld_in), coef f32 [4] = c1, c2, c3, c0:
+ * out act [T, F] = c1 z / rms(z) + c2 z^2 / rms(z^2) + c3 z^3 / rms(z^3) + c0, rms(u) = sqrt(mean_F(u^2) + eps), f32. */
+int lv_polynorm(const void* in, int64_t ld_in, const void* coef, void* out, int64_t T, int F, float eps, int dtype,
+                void* stream);
+
+/* in act [T, E*2F] (row stride ld_in), expert e's columns = [gate F | up F]; in_scale f32 [T, E] or NULL (all one);
+ * out_gate act, a scalar for each token at stride ld_gate, or NULL.
+ * s = in_scale[t, e]; g = min(s * gate, limit); u = clamp(s * up, -limit, limit);
+ * out act [T, E*F] (row stride ld_out) = g * sigmoid(alpha * g) * (u + 1) * sigmoid(out_gate[t]); 0 where s == 0. */
+int lv_expert_glu(const void* in, int64_t ld_in, const void* in_scale, const void* out_gate, int64_t ld_gate, void* out,
+                  int64_t ld_out, int64_t T, int E, int F, float limit, float alpha, int dtype, void* stream);
+
+/* lv_moe_grouped_ff for clamped gated experts: up_w bf16 [E*2F, W] (per expert F gate rows, then F up rows),
+ * down_w bf16 [W, E*F] with row stride down_ld (0: E*F; a column block of a wider weight otherwise).
+ * out[t] = sum_k W_down,e glu(weights[t, k] * W_gu,e h[t]), e = ids[t, k]: the weight scales the expert's input and the
+ * outputs are summed as they are. Workspace: lv_moe_grouped_workspace_bytes(T, W, F, E, top) bytes, 16-byte aligned. */
+int lv_moe_grouped_glu_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w,
+                          int64_t down_ld, void* out, void* workspace, int64_t T, int W, int F, int E, int top, float limit,
+                          float alpha, void* stream);
 
 #ifdef __cplusplus
 }

@@ -16,8 +16,9 @@ from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc", "mixers")
 LIB_PATH = os.path.join(_HERE, "lib", "liblvmix.so")
-SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip", "mix_latent.hip", "mix_moe_gemm.hip"]
-ABI_VERSION = 5
+SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip", "mix_latent.hip", "mix_moe_gemm.hip",
+           "mix_sandwich.hip"]
+ABI_VERSION = 6
 
 _P = c_void_p
 SIGNATURES = {
@@ -36,20 +37,27 @@ SIGNATURES = {
     "lv_pool_update": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                c_int, c_int, _P]),
     "lv_window_pool_attn": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int64, c_int,
-                                    c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int64, c_int64, c_int, _P]),
+                                    c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int64, c_int64, c_int, c_int, _P]),
     "lv_window_pool_attn_mfma": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int, c_int, c_int, c_int,
                                          c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P, c_int64,
-                                         c_int64, c_int64, _P]),
+                                         c_int64, c_int64, c_int, _P]),
     "lv_latent_prep": (c_int, [_P, c_int64, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int,
                                c_int, c_int, c_int, c_float, c_int, _P]),
     "lv_latent_q_finish": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     "lv_latent_out_gate": (c_int, [_P, _P, c_int64, c_int, _P, c_int64, c_int, c_int, c_int, _P]),
-    "lv_moe_route": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
+    "lv_moe_route": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P]),
     "lv_relu2_scale": (c_int, [_P, _P, _P, c_int64, c_int, c_int, c_int, _P]),
     "lv_moe_grouped_ff": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
     "lv_moe_grouped_workspace_bytes": (c_int64, [c_int64, c_int, c_int, c_int, c_int]),
     "lv_moe_sort": (c_int, [_P, c_int64, c_int, c_int, _P, _P, _P, _P]),
     "lv_moe_combine": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P]),
+    "lv_sandwich_add_norm": (c_int, [_P, _P, _P, _P, _P, _P, c_float, _P, c_int64, c_int, c_float, c_int, _P]),
+    "lv_rotary_store": (c_int, [_P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64,
+                                c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_polynorm": (c_int, [_P, c_int64, _P, _P, c_int64, c_int, c_float, c_int, _P]),
+    "lv_expert_glu": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, c_int64, c_int, c_int, c_float, c_float, c_int, _P]),
+    "lv_moe_grouped_glu_ff": (c_int, [_P, _P, _P, _P, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_float,
+                                      c_float, _P]),
 }
 
 _lib = None

@@ -11,7 +11,7 @@
 //   latent_q_finish_kernel  one workgroup per token: [absorbed query | rotated positional query part] per head.
 //   latent_out_gate_kernel  elementwise: head-major outputs to token-major rows times sigmoid(gate).
 //   moe_route_kernel        one wave per token: sigmoid scores, correction for the choice only, group limit, top-k,
-//                           normalised weights; the wave keeps its scores in LDS and picks maxima by shuffles.
+//                           normalised (or raw) weights; the wave keeps its scores in LDS and picks maxima by shuffles.
 //   relu2_scale_kernel      elementwise: relu(x)^2 times the token's weight for the expert the column belongs to.
 #include "mix_common.h"
 
@@ -133,7 +133,8 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                         int32_t* __restrict__ ids, float* __restrict__ weights,
-                                                        float* __restrict__ dense, int E, int top, int groups, int keep) {
+                                                        float* __restrict__ dense, int E, int top, int groups, int keep,
+                                                        int normalize) {
   extern __shared__ float rl[];
   float* s_lds = rl;              // [E] scores
   float* c_lds = rl + E;          // [E] selection scores, -inf once out of the running
@@ -195,7 +196,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     __syncthreads();
   }
   if (lane < top) {
-    const float w = mine / (wsum + 1e-20f);
+    const float w = normalize ? mine / (wsum + 1e-20f) : mine;
     ids[t * top + lane] = mine_id;
     weights[t * top + lane] = w;
     if (dense != nullptr) dense[t * E + mine_id] = w;
@@ -292,7 +293,7 @@ int lv_latent_out_gate(const void* o, const void* gate, int64_t ld_gate, int gat
 }
 
 int lv_moe_route(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
-                 int top, int groups, int keep, void* stream) {
+                 int top, int groups, int keep, int normalize, void* stream) {
   if (T == 0) return 0;
   if (!logits || !ids || !weights || T < 0 || E <= 0 || top <= 0 || top > E || top > kWave)
     return fail(-1, "lv_moe_route: bad arguments (experts %d, top %d)", E, top);
@@ -302,7 +303,7 @@ int lv_moe_route(const void* logits, const void* correction, void* ids, void* we
   if (shm > 64 * 1024) return fail(-2, "lv_moe_route: %d experts need %zu bytes of LDS", E, shm);
   moe_route_kernel<<<dim3(static_cast<unsigned>(T)), dim3(kWave), shm, as_stream(stream)>>>(
       static_cast<const float*>(logits), static_cast<const float*>(correction), static_cast<int32_t*>(ids),
-      static_cast<float*>(weights), static_cast<float*>(dense), E, top, groups, keep);
+      static_cast<float*>(weights), static_cast<float*>(dense), E, top, groups, keep, normalize);
   return launched("lv_moe_route");
 }
 

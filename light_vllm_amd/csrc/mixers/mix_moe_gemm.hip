@@ -10,7 +10,8 @@
 //                        (v_mfma_f32_16x16x32_bf16) are 16-byte loads straight from memory; the four waves share the
 //                        tile's rows and split its columns. The weights are the MFMA's first operand: a lane then holds
 //                        four consecutive columns of one row and stores them as 8 bytes.
-//                        UP: rows are gathered from the tokens' activations, epilogue relu(x)^2.
+//                        UP: rows are gathered from the tokens' activations, epilogue relu(x)^2, or (GLU) the clamped
+//                        gated unit of a gate and an up block of the same columns.
 //                        DOWN: rows are the sorted activations, B_e is a column block of the one [width, experts*ff] weight.
 //   moe_combine_kernel   one workgroup per token: sum over its choices of weight * expert output row, in f32.
 // A row's result does not depend on where the sort put it or on what else is in the tile: every output element is
@@ -79,6 +80,8 @@ struct MoeGemmParams {
   int N, K, top;
   int64_t lda, ldb, ldc;
   int64_t b_expert;        // elements from one expert's B to the next
+  const float* row_scale;  // GLU: [pairs] factor on the pre-activations of a (token, choice) pair
+  float limit, alpha;      // GLU: clamp and sigmoid slope of the gated unit
 };
 
 // MB x NB blocks of 16 x 16 per wave; WM waves along the rows (1 or 2), the others along the columns: the workgroup's
@@ -86,8 +89,14 @@ struct MoeGemmParams {
 // matrix instructions of the current one are issued, so that memory latency is covered by them. KU > 0 (tiles of a few
 // rows, where the weights are read once and the launch is bound by memory): the fragments of KU steps are requested
 // together instead, and many small workgroups keep the memory system full.
-template <int MB, int NB, int WM, bool UP, int KU = 0>
+// GLU (with UP; NB even): an expert's B holds N gate rows followed by N up rows; blocks 2c and 2c + 1 of a wave are the
+// gate and the up pre-activations of the SAME 16 columns, so the gated unit
+//   g = min(s * gate, L); u = clamp(s * up, -L, L); y = g * sigmoid(alpha * g) * (u + 1),  s = row_scale[pair of the row]
+// is formed in registers and one N-wide row is stored.
+template <int MB, int NB, int WM, bool UP, int KU = 0, bool GLU = false>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
+  static_assert(!GLU || (UP && NB % 2 == 0), "the gated unit pairs column blocks of the up projection");
+  constexpr int CB = GLU ? NB / 2 : NB;             // distinct 16-column blocks of a wave
   const int tile = blockIdx.y, bx = blockIdx.x;
   if (tile >= p.num_tiles[0]) return;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
   const int wm = wave % WM, wn = wave / WM;
   const int e = p.tiles[3 * tile], row0 = p.tiles[3 * tile + 1], nrows = p.tiles[3 * tile + 2];
   const int m0 = wm * 16 * MB;
-  const int n0 = (bx * (4 / WM) + wn) * 16 * NB;
+  const int n0 = (bx * (4 / WM) + wn) * 16 * CB;
   if (n0 >= p.N || m0 >= nrows) return;
   const uint16_t* arow[MB];
 #pragma unroll
@@ -107,7 +116,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
   const uint16_t* brow[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    const int n = min(n0 + nb * 16 + ln, p.N - 1);
+    const int n = min(n0 + (GLU ? nb / 2 : nb) * 16 + ln, p.N - 1) + (GLU && (nb & 1) ? p.N : 0);
     brow[nb] = p.B + static_cast<int64_t>(e) * p.b_expert + static_cast<int64_t>(n) * p.ldb + 8 * lg;
   }
   f32x4_t acc[MB][NB];
@@ -155,17 +164,26 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
     const int r = m0 + mb * 16 + ln;
     if (r >= nrows) continue;
     uint16_t* crow = p.C + static_cast<int64_t>(row0 + r) * p.ldc;
+    float rs = 1.0f;
+    if constexpr (GLU) rs = p.row_scale[p.sorted_pair[row0 + r]];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
+    for (int nb = 0; nb < CB; ++nb) {
       const int n = n0 + nb * 16 + 4 * lg;
       if (n >= p.N) continue;                                   // N is a multiple of 4: a lane's four columns are in or out together
       uint16_t o[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = acc[mb][nb][i];
-        if (UP) {
-          v = fmaxf(v, 0.0f);
-          v = v * v;
+        float v;
+        if constexpr (GLU) {
+          const float g = fminf(acc[mb][2 * nb][i] * rs, p.limit);
+          const float u = fminf(fmaxf(acc[mb][2 * nb + 1][i] * rs, -p.limit), p.limit);
+          v = g * sigmoidf_(p.alpha * g) * (u + 1.0f);
+        } else {
+          v = acc[mb][nb][i];
+          if (UP) {
+            v = fmaxf(v, 0.0f);
+            v = v * v;
+          }
         }
         bf16_t t;
         stf(&t, v);
@@ -184,7 +202,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __rest
   for (int c = threadIdx.x * 4; c < W; c += blockDim.x * 4) {
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int k = 0; k < top; ++k) {
-      const float w = weights[t * top + k];
+      const float w = weights != nullptr ? weights[t * top + k] : 1.0f;
       const uint2 v = *reinterpret_cast<const uint2*>(rows + static_cast<int64_t>(inv[t * top + k]) * W + c);
       acc[0] += w * __builtin_bit_cast(float, v.x << 16);
       acc[1] += w * __builtin_bit_cast(float, v.x & 0xffff0000u);
@@ -199,17 +217,19 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __rest
   }
 }
 
-template <bool UP>
+template <bool UP, bool GLU = false>
 static void gemm_launch(const MoeGemmParams& p, int max_tiles, int BM, hipStream_t s) {
-  if (BM == 128) {                 // 128 rows x 128 columns
-    dim3 grid((p.N + 127) / 128, max_tiles);
-    moe_gemm_kernel<4, 4, 2, UP><<<grid, dim3(256), 0, s>>>(p);
-  } else if (BM == 64) {           // 64 rows x 256 columns
-    dim3 grid((p.N + 255) / 256, max_tiles);
-    moe_gemm_kernel<4, 4, 1, UP><<<grid, dim3(256), 0, s>>>(p);
+  if (BM == 128) {                 // 128 rows x 128 columns (gated: 64, each from a gate and an up block)
+    const int cols = GLU ? 64 : 128;
+    dim3 grid((p.N + cols - 1) / cols, max_tiles);
+    moe_gemm_kernel<4, 4, 2, UP, 0, GLU><<<grid, dim3(256), 0, s>>>(p);
+  } else if (BM == 64) {           // 64 rows x 256 columns (gated: 128)
+    const int cols = GLU ? 128 : 256;
+    dim3 grid((p.N + cols - 1) / cols, max_tiles);
+    moe_gemm_kernel<4, 4, 1, UP, 0, GLU><<<grid, dim3(256), 0, s>>>(p);
   } else {                         // 16 rows x 64 columns, four steps over k requested at once
     dim3 grid((p.N + 63) / 64, max_tiles);
-    moe_gemm_kernel<1, 1, 1, UP, 4><<<grid, dim3(256), 0, s>>>(p);
+    moe_gemm_kernel<1, GLU ? 2 : 1, 1, UP, 4, GLU><<<grid, dim3(256), 0, s>>>(p);
   }
 }
 
@@ -256,14 +276,51 @@ int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const
   moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, s>>>(static_cast<const int32_t*>(ids), static_cast<int>(M), E, BM,
                                                           sorted_pair, inv, tiles, num_tiles, max_tiles, nullptr, 1);
   MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act, sorted_pair, tiles, num_tiles,
-                   F, W, top, W, W, F, static_cast<int64_t>(F) * W};
+                   F, W, top, W, W, F, static_cast<int64_t>(F) * W, nullptr, 0.0f, 0.0f};
   gemm_launch<true>(up, max_tiles, BM, s);
   MoeGemmParams down{act, static_cast<const uint16_t*>(down_w), rows, sorted_pair, tiles, num_tiles,
-                     W, F, top, F, static_cast<int64_t>(E) * F, W, F};
+                     W, F, top, F, static_cast<int64_t>(E) * F, W, F, nullptr, 0.0f, 0.0f};
   gemm_launch<false>(down, max_tiles, BM, s);
   moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, static_cast<const float*>(weights),
                                                                           static_cast<uint16_t*>(out), W, top);
   return launched("lv_moe_grouped_ff");
+}
+
+int lv_moe_grouped_glu_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w,
+                          int64_t down_ld, void* out, void* workspace, int64_t T, int W, int F, int E, int top, float limit,
+                          float alpha, void* stream) {
+  if (T == 0) return 0;
+  if (!h || !ids || !weights || !up_w || !down_w || !out || !workspace) return fail(-1, "lv_moe_grouped_glu_ff: null pointer");
+  if (T < 0 || W <= 0 || F <= 0 || E <= 0 || top <= 0 || W % 32 != 0 || F % 32 != 0 || E > 4096)
+    return fail(-1, "lv_moe_grouped_glu_ff: width %d and expert size %d must be multiples of 32 (experts %d)", W, F, E);
+  if (down_ld <= 0) down_ld = static_cast<int64_t>(E) * F;
+  if (down_ld < static_cast<int64_t>(E) * F || down_ld % 8 != 0 || (reinterpret_cast<uintptr_t>(down_w) & 15) != 0 ||
+      (reinterpret_cast<uintptr_t>(up_w) & 15) != 0 || (reinterpret_cast<uintptr_t>(h) & 15) != 0)
+    return fail(-1, "lv_moe_grouped_glu_ff: row stride or alignment of the weights");
+  const int64_t M = T * top;
+  if (M > (1 << 30)) return fail(-2, "lv_moe_grouped_glu_ff: %lld rows", (long long)M);
+  const int BM = lv_moe_tile_rows(M, E);
+  const int max_tiles = lv_moe_max_tiles(M, E, BM);
+  // workspace as in lv_moe_grouped_ff
+  int32_t* sorted_pair = static_cast<int32_t*>(workspace);
+  int32_t* inv = sorted_pair + M;
+  int32_t* tiles = inv + M;
+  int32_t* num_tiles = tiles + 3 * static_cast<int64_t>(max_tiles);
+  const int64_t ints = (2 * M + 3 * static_cast<int64_t>(max_tiles) + 1 + 3) / 4 * 4;
+  uint16_t* act = reinterpret_cast<uint16_t*>(sorted_pair + ints);
+  uint16_t* rows = act + M * F;
+  hipStream_t s = as_stream(stream);
+  const size_t shm = sizeof(int32_t) * (3 * static_cast<size_t>(E) + 2);
+  moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, s>>>(static_cast<const int32_t*>(ids), static_cast<int>(M), E, BM,
+                                                          sorted_pair, inv, tiles, num_tiles, max_tiles, nullptr, 1);
+  MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act, sorted_pair, tiles, num_tiles,
+                   F, W, top, W, W, F, 2 * static_cast<int64_t>(F) * W, static_cast<const float*>(weights), limit, alpha};
+  gemm_launch<true, true>(up, max_tiles, BM, s);
+  MoeGemmParams down{act, static_cast<const uint16_t*>(down_w), rows, sorted_pair, tiles, num_tiles,
+                     W, F, top, F, down_ld, W, F, nullptr, 0.0f, 0.0f};
+  gemm_launch<false>(down, max_tiles, BM, s);
+  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, nullptr, static_cast<uint16_t*>(out), W, top);
+  return launched("lv_moe_grouped_glu_ff");
 }
 
 int lv_moe_sort(const void* ids, int64_t M, int E, int align, void* sorted_pair, void* inv, void* offsets, void* stream) {
@@ -279,7 +336,7 @@ int lv_moe_sort(const void* ids, int64_t M, int E, int align, void* sorted_pair,
 
 int lv_moe_combine(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top, void* stream) {
   if (T == 0) return 0;
-  if (!rows || !inv || !weights || !out || T < 0 || W <= 0 || W % 4 != 0 || top <= 0) return fail(-1, "lv_moe_combine: bad arguments");
+  if (!rows || !inv || !out || T < 0 || W <= 0 || W % 4 != 0 || top <= 0) return fail(-1, "lv_moe_combine: bad arguments");
   moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, as_stream(stream)>>>(
       static_cast<const uint16_t*>(rows), static_cast<const int32_t*>(inv), static_cast<const float*>(weights),
       static_cast<uint16_t*>(out), W, top);

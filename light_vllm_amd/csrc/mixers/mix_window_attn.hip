@@ -79,6 +79,7 @@ __global__ __launch_bounds__(256) void pool_update_kernel(const T* __restrict__ 
 struct WindowAttnParams {
   const void *q, *k_cache, *v_cache, *kp, *vp, *gate;
   int64_t ld_gate;
+  int gate_dv;          // entries of a gate row per head: Dv (one per output channel) or 1 (one per head)
   void* out;
   const int32_t *cu_q, *ctx_lens, *tok_seq, *block_tables;
   int bt_stride, H, G, D, Dv, page, window, P, PP;
@@ -223,7 +224,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
       acc += o_lds[(w * kMaxRep + h) * Dv + dv] * c;
     }
     float r = ll > 0.0f ? acc / ll : 0.0f;
-    if (gate != nullptr) r *= sigmoidf_(ldf(gate + static_cast<int64_t>(h0 + h) * Dv + dv));
+    if (gate != nullptr) r *= sigmoidf_(ldf(gate + static_cast<int64_t>(h0 + h) * p.gate_dv + (p.gate_dv > 1 ? dv : 0)));
     stf(out + static_cast<int64_t>(h0 + h) * Dv + dv, r);
   }
 }
@@ -287,7 +288,7 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
                         const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
                         const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G, int D,
                         int Dv, int page, int window, int P, float scale, int has_sink, int64_t k_ld, int64_t v_ld,
-                        int dtype, void* stream) {
+                        int gate_kind, int dtype, void* stream) {
   if (T == 0) return 0;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !tok_seq || !block_tables)
     return fail(-1, "lv_window_pool_attn: null pointer");
@@ -298,10 +299,14 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
   if (T < 0 || H <= 0 || G <= 0 || H % G != 0 || D <= 0 || Dv <= 0 || page <= 0 || window <= 0 || bt_stride <= 0)
     return fail(-1, "lv_window_pool_attn: bad sizes");
   if (Dv > 8 * kWave) return fail(-2, "lv_window_pool_attn: value size %d above %d", Dv, 8 * kWave);
+  if (gate_kind != LV_MIX_GATE_PER_HEAD && gate_kind != LV_MIX_GATE_PER_CHANNEL)
+    return fail(-1, "lv_window_pool_attn: gate kind %d", gate_kind);
+  const int gate_dv = gate_kind == LV_MIX_GATE_PER_HEAD ? 1 : Dv;
+  if (gate != nullptr && ld_gate < static_cast<int64_t>(H) * gate_dv) return fail(-1, "lv_window_pool_attn: gate stride");
   const bool wide = Dv > 4 * kWave;
   const int kMaxRep = wide ? 4 : 8;
   const int rep = H / G;
-  WindowAttnParams p{q, k_cache, v_cache, kp, vp, gate, ld_gate, out, cu_q, ctx_lens, tok_seq, block_tables,
+  WindowAttnParams p{q, k_cache, v_cache, kp, vp, gate, ld_gate, gate_dv, out, cu_q, ctx_lens, tok_seq, block_tables,
                      bt_stride, H, G, D, Dv, page, window, P, P > 0 ? (page + P - 1) / P : 0, scale,
                      has_sink ? 1.0f : 0.0f, k_ld, v_ld, has_sink ? 0.0f : -1e30f};
   const size_t shm = sizeof(float) * (static_cast<size_t>(kMaxRep) * D + 4 * kMaxRep * kWave +

@@ -25,6 +25,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 struct WindowMfmaParams {
   const uint16_t *q, *k_cache, *v_cache, *kp, *vp, *gate;
   int64_t ld_gate;
+  int gate_dv;         // entries of a gate row per head: Dv (one per output channel) or 1 (one per head)
   uint16_t* out;
   const int32_t *cu_q, *ctx_lens, *block_tables;
   int bt_stride, H, G, D, Dv, page, window, P, PP, ngroups;
@@ -306,7 +307,8 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
   }
   const float inv = l > 0.0f ? 1.0f / l : 0.0f;
   uint16_t* orow = p.out + (t * p.H + h) * Dv;
-  const uint16_t* grow = p.gate != nullptr ? p.gate + t * p.ld_gate + static_cast<int64_t>(h) * Dv : nullptr;
+  const uint16_t* grow = p.gate != nullptr ? p.gate + t * p.ld_gate + static_cast<int64_t>(h) * p.gate_dv : nullptr;
+  const int gstep = p.gate_dv > 1 ? 1 : 0;
 #pragma unroll
   for (int d = 0; d < DVB; ++d) {
     if (d < ndvb) {
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
       for (int i = 0; i < 4; ++i) {
         const int dv = 16 * d + 4 * lg + i;
         float val = acc_o[d][i] * inv;
-        if (grow != nullptr) val *= sigmoidf_(__builtin_bit_cast(float, static_cast<uint32_t>(grow[dv]) << 16));
+        if (grow != nullptr) val *= sigmoidf_(__builtin_bit_cast(float, static_cast<uint32_t>(grow[dv * gstep]) << 16));
         orow[dv] = static_cast<uint16_t>(bf16_bits(val));
       }
     }
@@ -323,8 +325,8 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
 
 // One wave per (token, query head): combines the splits' partials (each with its own running maximum), applies the gate.
 __global__ __launch_bounds__(256) void window_pool_merge_kernel(const float* __restrict__ ws, const uint16_t* __restrict__ gate,
-                                                                int64_t ld_gate, uint16_t* __restrict__ out, int64_t items,
-                                                                int H, int Dv, int nsplit, float m0) {
+                                                                int64_t ld_gate, int gate_dv, uint16_t* __restrict__ out,
+                                                                int64_t items, int H, int Dv, int nsplit, float m0) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;
   if (item >= items) return;
@@ -341,7 +343,8 @@ __global__ __launch_bounds__(256) void window_pool_merge_kernel(const float* __r
     for (int s = 0; s < nsplit; ++s) acc += w[s * (Dv + 4) + dv] * expf(w[s * (Dv + 4) + Dv] - mm);
     float val = acc * inv;
     if (gate != nullptr)
-      val *= sigmoidf_(__builtin_bit_cast(float, static_cast<uint32_t>(gate[t * ld_gate + static_cast<int64_t>(h) * Dv + dv]) << 16));
+      val *= sigmoidf_(__builtin_bit_cast(float, static_cast<uint32_t>(gate[t * ld_gate + static_cast<int64_t>(h) * gate_dv +
+                                                                            (gate_dv > 1 ? dv : 0)]) << 16));
     out[item * Dv + dv] = static_cast<uint16_t>(bf16_bits(val));
   }
 }
@@ -357,7 +360,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                                         const int32_t* ctx_lens, const int32_t* block_tables, int bt_stride, int B,
                                         int max_new_tokens, int H, int G, int D, int Dv, int page, int window, int P,
                                         float scale, int has_sink, int nsplit, void* workspace, int64_t T, int64_t k_ld,
-                                        int64_t v_ld, void* stream) {
+                                        int64_t v_ld, int gate_kind, void* stream) {
   if (B == 0 || max_new_tokens <= 0) return 0;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !block_tables)
     return fail(-1, "lv_window_pool_attn_mfma: null pointer");
@@ -366,7 +369,10 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
     return fail(-1, "lv_window_pool_attn_mfma: bad sizes");
   if (D % 16 != 0 || Dv % 16 != 0 || D <= 0 || Dv <= 0 || D > 32 * kMaxK32 || Dv > 16 * kMaxDvb)
     return fail(-2, "lv_window_pool_attn_mfma: head sizes %d / %d (multiples of 16 up to 256)", D, Dv);
-  if (gate != nullptr && ld_gate < static_cast<int64_t>(H) * Dv) return fail(-1, "lv_window_pool_attn_mfma: gate stride");
+  if (gate_kind != LV_MIX_GATE_PER_HEAD && gate_kind != LV_MIX_GATE_PER_CHANNEL)
+    return fail(-1, "lv_window_pool_attn_mfma: gate kind %d", gate_kind);
+  const int gate_dv = gate_kind == LV_MIX_GATE_PER_HEAD ? 1 : Dv;
+  if (gate != nullptr && ld_gate < static_cast<int64_t>(H) * gate_dv) return fail(-1, "lv_window_pool_attn_mfma: gate stride");
   if (k_ld <= 0) k_ld = static_cast<int64_t>(G) * D;
   if (v_ld <= 0) v_ld = static_cast<int64_t>(G) * Dv;
   if (k_ld < static_cast<int64_t>(G) * D || v_ld < static_cast<int64_t>(G) * Dv || k_ld % 8 != 0 || v_ld % 4 != 0 ||
@@ -377,7 +383,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
   const int ngroups = (rep + 3) / 4;
   WindowMfmaParams p{static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(k_cache),
                      static_cast<const uint16_t*>(v_cache), static_cast<const uint16_t*>(kp),
-                     static_cast<const uint16_t*>(vp), static_cast<const uint16_t*>(gate), ld_gate,
+                     static_cast<const uint16_t*>(vp), static_cast<const uint16_t*>(gate), ld_gate, gate_dv,
                      static_cast<uint16_t*>(out), cu_q, ctx_lens, block_tables, bt_stride, H, G, D, Dv, page, window, P,
                      P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f,
                      magic(page), magic(P > 0 ? P : 1), magic(Dv / 4), nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace),
@@ -398,8 +404,8 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
   if (nsplit > 1) {
     const int64_t items = T * H;
     window_pool_merge_kernel<<<dim3(static_cast<unsigned>((items + 3) / 4)), block, 0, st>>>(
-        static_cast<const float*>(workspace), static_cast<const uint16_t*>(gate), ld_gate, static_cast<uint16_t*>(out),
-        items, H, Dv, nsplit, m0);
+        static_cast<const float*>(workspace), static_cast<const uint16_t*>(gate), ld_gate, gate_dv,
+        static_cast<uint16_t*>(out), items, H, Dv, nsplit, m0);
   }
   return launched("lv_window_pool_attn_mfma");
 }

@@ -1,5 +1,6 @@
 """SwiGLU: silu(gate) * up over the two halves of the last dim (reference "native" backend,
-lightvllm/layers/activation.py:7-29), and the clamped gated unit with a sigmoid of slope alpha."""
+lightvllm/layers/activation.py:7-29), the clamped gated unit with a sigmoid of slope alpha, and PolyNorm,
+a learned cubic of the row-normalised powers of its input."""
 import torch
 import torch.nn.functional as F
 from torch import nn
@@ -26,3 +27,16 @@ class ClampedGLU(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return mix_ops.clamped_glu(x, self.limit, self.alpha)
+
+
+class PolyNorm(nn.Module):
+    """c1 R(z) + c2 R(z^2) + c3 R(z^3) + c0 over the last dim, powers element by element, R(u) = u / sqrt(mean(u^2) + eps)
+    per token; coef = (c1, c2, c3, c0), f32."""
+
+    def __init__(self, eps: float = 1e-6):
+        super().__init__()
+        self.eps = float(eps)
+        self.coef = nn.Parameter(torch.tensor([1.0, 0.0, 0.0, 0.0], dtype=torch.float32))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return mix_ops.polynorm(x, self.coef, self.eps)

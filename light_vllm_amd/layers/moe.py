@@ -22,6 +22,16 @@ matrices one [width, experts * ff] weight. Two forms compute the same sum:
     experts / top times the FLOPs of the gathered form.
 
 The gathered and masked forms never synchronise with the host, so both can be captured into a hipGraph.
+
+GLUSparseMoE is the same mixture with clamped gated experts (gate and up matrices), a router without correction
+or groups whose weights are the chosen scores themselves, the weight applied to the expert's INPUT,
+    y = sum_chosen expert_e(s_e * h),    expert(x) = W_down [min(W_gate x, L) * sigmoid(alpha min(W_gate x, L)) * (clamp(W_up x, -L, L) + 1)]
+and an optional shared expert of the same form that every token uses, times sigmoid(w_sg . h). Because the
+projections are linear, s * h enters as a factor on the pre-activations (mix_ops.expert_glu), and the shared
+expert's token gate as a factor on its activations, so all of it is GEMMs on h plus one elementwise kernel.
+Forms: masked (everything in one up GEMM and one down GEMM; any dtype and size) and gathered (bf16: sort, two
+grouped GEMMs on the matrix cores with the gated unit in the first one's epilogue, sum; the shared expert as
+vendor GEMMs beside it).
 """
 from __future__ import annotations
 
@@ -80,3 +90,48 @@ class SparseMoE(nn.Module):
             return mix_ops.moe_sorted_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff)
         up = F.linear(h, self.up_weight)
         return F.linear(mix_ops.relu2_scale(up, dense, self.E, self.ff), self.down_weight)
+
+
+class GLUSparseMoE(nn.Module):
+    """Weights: up_weight [E*2*ff + 2*shared_ff + 1, width] = per expert [gate | up] rows, then the shared
+    expert's gate and up rows and the row of its token gate; down_weight [width, E*ff + shared_ff]."""
+
+    def __init__(self, width: int, ff: int, experts: int, top: int, limit: float, alpha: float = 1.702,
+                 shared_ff: int = 0, shared_limit: float = 0.0):
+        super().__init__()
+        assert tp_size() == 1, "the mixture of experts is not sharded: run it with tensor_parallel_size 1"
+        assert 1 <= top <= experts and shared_ff >= 0
+        self.width, self.ff, self.E, self.top = width, ff, experts, top
+        self.limit, self.alpha, self.Fs, self.shared_limit = float(limit), float(alpha), shared_ff, float(shared_limit)
+        self.router_weight = nn.Parameter(torch.empty(experts, width, dtype=torch.float32))
+        self.up_weight = nn.Parameter(torch.empty(experts * 2 * ff + (2 * shared_ff + 1 if shared_ff else 0), width))
+        self.down_weight = nn.Parameter(torch.empty(width, experts * ff + shared_ff))
+
+    def route(self, h: torch.Tensor):
+        logits = F.linear(h.float(), self.router_weight)
+        return mix_ops.moe_route(logits, None, self.top, 1, 1, normalize=False)
+
+    def form(self, h: torch.Tensor) -> str:
+        if MOE_KERNEL in ("masked", "gathered"):
+            return MOE_KERNEL
+        ok = mix_ops.moe_grouped_ok(h, self.ff) and (self.E * self.ff + self.Fs) % 8 == 0
+        return "gathered" if ok and self.E >= GATHER_FROM * self.top else "masked"
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        ids, weights, dense = self.route(h)
+        E, Fe, Fs, T = self.E, self.ff, self.Fs, h.size(0)
+        if self.form(h) == "gathered":
+            routed_down = self.down_weight[:, :E * Fe]
+            y = mix_ops.moe_grouped_glu_ff(h, ids, weights, self.up_weight[:E * 2 * Fe], routed_down, E, Fe, self.limit, self.alpha)
+            if Fs:
+                up = F.linear(h, self.up_weight[E * 2 * Fe:])
+                a = mix_ops.expert_glu(up[:, :2 * Fs], 1, Fs, self.shared_limit, self.alpha, out_gate=up[:, 2 * Fs])
+                y = torch.addmm(y, a, self.down_weight[:, E * Fe:].t())
+            return y
+        up = F.linear(h, self.up_weight)
+        act = torch.empty(T, E * Fe + Fs, dtype=h.dtype, device=h.device)
+        mix_ops.expert_glu(up[:, :E * 2 * Fe], E, Fe, self.limit, self.alpha, in_scale=dense, out=act[:, :E * Fe])
+        if Fs:
+            mix_ops.expert_glu(up[:, E * 2 * Fe:E * 2 * Fe + 2 * Fs], 1, Fs, self.shared_limit, self.alpha,
+                               out_gate=up[:, E * 2 * Fe + 2 * Fs], out=act[:, E * Fe:])
+        return F.linear(act, self.down_weight)

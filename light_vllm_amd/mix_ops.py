@@ -86,6 +86,90 @@ def residual_add_norm(x, y1=None, y2=None, w=None, w_offset=0.0, eps=1e-6, act_d
     return out
 
 
+def sandwich_add_norm(x, y=None, post_w=None, rows=None, vec=None, w=None, w_offset=1.0, eps=1e-6, act_dtype=None):
+    """The residual update of a layer that norms each sublayer's output as well as its input, fused with
+    what follows it. x [T, W] f32, in place:
+        x += y / sqrt(mean(y^2) + eps) * (w_offset + post_w)      (y act [T, W]; skipped when y is None)
+        x += rows + vec                                            (rows act [T, W], vec f32 [W]; either may be None)
+    and returns x / sqrt(mean(x^2) + eps) * (w_offset + w) in act dtype (None when w is None). All sums and
+    both norms are f32."""
+    T, W = x.shape
+    _f32(x, post_w, vec, w)
+    assert (y is None) == (post_w is None)
+    act_dtype = act_dtype or next((t.dtype for t in (y, rows) if t is not None), torch.bfloat16)
+    out = torch.empty(T, W, dtype=act_dtype, device=x.device) if w is not None else None
+    if x.is_cuda:
+        for t in (y, rows):
+            assert t is None or (t.is_contiguous() and t.dtype == act_dtype and t.shape == (T, W))
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_sandwich_add_norm(_p(x), _p(y), _p(post_w), _p(rows), _p(vec), _p(w), w_offset, _p(out), T, W,
+                                               eps, _DT[act_dtype], _stream(x)), "lv_sandwich_add_norm")
+        return out
+    if y is not None:
+        yf = y.float()
+        x.add_(yf / torch.sqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * (w_offset + post_w))
+    if rows is not None:
+        x.add_(rows.float())
+    if vec is not None:
+        x.add_(vec)
+    if w is None:
+        return None
+    out.copy_(x / torch.sqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (w_offset + w))
+    return out
+
+
+def polynorm(z, coef, eps):
+    """z act [T, F] -> act [T, F] = c1 R(z) + c2 R(z^2) + c3 R(z^3) + c0 with coef = (c1, c2, c3, c0) f32 [4], powers
+    element by element and R(u) = u / sqrt(mean_F(u^2) + eps) per token, in f32."""
+    T, Fd = z.shape
+    _f32(coef)
+    out = torch.empty(T, Fd, dtype=z.dtype, device=z.device)
+    if z.is_cuda:
+        assert z.stride(1) == 1 and coef.numel() == 4
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_polynorm(_p(z), z.stride(0), _p(coef), _p(out), T, Fd, eps, _DT[z.dtype], _stream(z)), "lv_polynorm")
+        return out
+    zf = z.float()
+    acc = coef[3].expand_as(zf).clone()
+    for k in range(3):
+        u = zf.pow(k + 1)
+        acc = acc + coef[k] * u / torch.sqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    out.copy_(acc)
+    return out
+
+
+def expert_glu(x, E, Fe, limit, alpha, in_scale=None, out_gate=None, out=None):
+    """Clamped gated unit of E experts side by side. x act [T, E*2*Fe] (row stride free), expert e's columns
+    [gate Fe | up Fe]. With in_scale f32 [T, E] the pre-activations are multiplied by in_scale[t, e] first (the
+    expert ran on its input times that number; an expert whose number is 0 gives zeros). With out_gate (act [T],
+    any stride) the result is multiplied by sigmoid(out_gate[t]).
+        g = min(s * gate, L); u = clamp(s * up, -L, L); y = g * sigmoid(alpha * g) * (u + 1)
+    Writes act [T, E*Fe] into `out` (a view with free row stride) or a new tensor; returns it."""
+    T = x.size(0)
+    assert x.size(1) == E * 2 * Fe and x.stride(1) == 1
+    if out is None:
+        out = torch.empty(T, E * Fe, dtype=x.dtype, device=x.device)
+    assert out.shape == (T, E * Fe) and out.stride(1) == 1 and out.dtype == x.dtype
+    if x.is_cuda:
+        assert in_scale is None or (in_scale.dtype == torch.float32 and in_scale.is_contiguous() and in_scale.shape == (T, E))
+        assert out_gate is None or (out_gate.dtype == x.dtype and out_gate.shape == (T,))
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_expert_glu(_p(x), x.stride(0), _p(in_scale), _p(out_gate), out_gate.stride(0) if out_gate is not None else 0,
+                                        _p(out), out.stride(0), T, E, Fe, limit, alpha, _DT[x.dtype], _stream(x)), "lv_expert_glu")
+        return out
+    xe = x.float().view(T, E, 2, Fe)
+    sc = in_scale.view(T, E, 1) if in_scale is not None else 1.0
+    g = (xe[:, :, 0] * sc).clamp(max=limit)
+    u = (xe[:, :, 1] * sc).clamp(-limit, limit)
+    yv = g * torch.sigmoid(alpha * g) * (u + 1)
+    if in_scale is not None:
+        yv = torch.where(in_scale.view(T, E, 1) != 0, yv, torch.zeros_like(yv))
+    if out_gate is not None:
+        yv = yv * torch.sigmoid(out_gate.float()).view(T, 1, 1)
+    out.copy_(yv.reshape(T, E * Fe))
+    return out
+
+
 def clamped_glu(x, limit: float, alpha: float):
     """x [T, 2F] = [gate | up] -> min(g, L) * sigmoid(alpha * g) * (clamp(u, -L, L) + 1), [T, F]."""
     T, F2 = x.shape
@@ -310,10 +394,12 @@ def pool_update(k_cache, v_cache, kp, vp, step, G, D, Dv, P):
             vpf[dst] = vc[rows].float().mean(0)
 
 
-def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, window, P, scale, has_sink=True):
+def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, window, P, scale, has_sink=True,
+                          gate_per_head=False):
     """Query at position i attends to cached positions j with 0 <= i - j < window and to the pooled
     entry of every block b with b*P + P - 1 <= i - window, one softmax over both, `has_sink` adding 1
-    to its denominator; the result is multiplied by sigmoid(gate) when a gate is given.
+    to its denominator; the result is multiplied by sigmoid(gate) when a gate is given (gate rows hold
+    H*Dv numbers, one per output channel, or H with `gate_per_head`).
     q [T, H*D] contiguous act; returns act [T, H*Dv]. k_cache and v_cache [pages, page, G, D|Dv] may be
     views of wider token rows (one cache row serving as key and, in part, as value). A window that no
     sequence reaches, no pool and no sink give plain causal softmax attention."""
@@ -322,7 +408,7 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
     k_ld, v_ld = k_cache.stride(1), v_cache.stride(1)
     if q.is_cuda:
-        assert q.is_contiguous() and (gate is None or gate.stride(1) == 1)
+        assert q.is_contiguous() and (gate is None or (gate.stride(1) == 1 and gate.size(1) == (H if gate_per_head else H * Dv)))
         for c, ld, d in ((k_cache, k_ld, D), (v_cache, v_ld, Dv)):
             assert c.stride(3) == 1 and (G == 1 or c.stride(2) == d) and c.stride(0) == page * ld and ld >= G * d
         lib = _mixlib.load()
@@ -344,14 +430,16 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
                                                        _p(step.ctx_lens), _p(step.block_tables),
                                                        step.block_tables.stride(0), len(step.host_lens_q),
                                                        max(step.host_lens_q), H, G, D, Dv, page, window, P, scale,
-                                                       int(has_sink), nsplit, _p(ws), T, k_ld, v_ld, _stream(q)),
+                                                       int(has_sink), nsplit, _p(ws), T, k_ld, v_ld, 0 if gate_per_head else 1,
+                                                       _stream(q)),
                           "lv_window_pool_attn_mfma")
             return out
         _mixlib.check(lib.lv_window_pool_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
                                               gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
                                               _p(step.ctx_lens), _p(step.tok_seq), _p(step.block_tables),
                                               step.block_tables.stride(0), T, H, G, D, Dv, page, window, P, scale,
-                                              int(has_sink), k_ld, v_ld, _DT[q.dtype], _stream(q)), "lv_window_pool_attn")
+                                              int(has_sink), k_ld, v_ld, 0 if gate_per_head else 1, _DT[q.dtype], _stream(q)),
+                      "lv_window_pool_attn")
         return out
     PP = pooled_slots(page, P)
     rep = H // G
@@ -377,17 +465,28 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
             w = e / (e.sum(-1, keepdim=True) + (torch.exp(-m) if has_sink else 0))
             o = torch.einsum("grn,ngv->grv", w, V).reshape(H * Dv)
             if gate is not None:
-                o = o * torch.sigmoid(gate[q0 + r].float())
+                gr = torch.sigmoid(gate[q0 + r].float())
+                o = o * (gr.repeat_interleave(Dv) if gate_per_head else gr)
             out[q0 + r] = o
         q0 += n
     return out
 
 
 # ------------------------------------------------------------------------------- latent attention
-def rotary_inv_freq(dims: int, base: float, device) -> torch.Tensor:
-    """f32 [dims/2]: base^(-2i/dims), computed in 64-bit and rounded once."""
+def rotary_inv_freq(dims: int, base: float, device, scaling: dict | None = None) -> torch.Tensor:
+    """f32 [dims/2]: base^(-2i/dims), computed in 64-bit and rounded once. `scaling` (factor, low, high,
+    original) rescales by wavelength 2 pi / f: waves shorter than original / high keep their frequency,
+    waves longer than original / low get f / factor, and those between are blended linearly in
+    original / wavelength."""
     i = torch.arange(dims // 2, dtype=torch.float64)
-    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    if scaling:
+        factor, low, high = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+        turns = float(scaling["original"]) * f / (2.0 * torch.pi)          # original / wavelength
+        blend = ((turns - low) / (high - low)).clamp(0.0, 1.0) if high != low else (turns >= high).double()
+        blend = torch.where(turns > high, torch.ones_like(blend), torch.where(turns < low, torch.zeros_like(blend), blend))
+        f = (1.0 - blend) * f / factor + blend * f
+    return f.float().to(device)
 
 
 def _rotate(x, pos, inv_freq, dims):
@@ -403,6 +502,45 @@ def _rotate(x, pos, inv_freq, dims):
 
 def _positions(step, device):
     return torch.cat([torch.arange(c, c + n, device=device) for n, c in zip(step.host_lens_q, step.host_ctx_lens)])
+
+
+def rotary_store(proj, off_q, off_k, off_v, inv_freq, head_scale, k_cache, v_cache, step, H, G, D, Dv, rot_dims):
+    """proj act [T, ld]: queries at column off_q (H heads of D), keys at off_k (G heads of D), values at off_v
+    (G heads of Dv). The first rot_dims entries of every query and key head are rotated (entry i pairs with
+    i + rot_dims/2, angle = position * inv_freq[i], f32); each query head is then multiplied by head_scale[h]
+    (f32 [H], may be None). Rotated keys and the values go to the token's row of the paged caches
+    [pages, page, G, D|Dv]. Returns the queries, act [T, H*D]."""
+    T = proj.size(0)
+    page = k_cache.size(1)
+    _f32(inv_freq, head_scale)
+    q_out = torch.empty(T, H * D, dtype=proj.dtype, device=proj.device)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == proj.dtype and v_cache.dtype == proj.dtype
+    assert 0 <= rot_dims <= D and rot_dims % 2 == 0 and (rot_dims == 0 or inv_freq.numel() == rot_dims // 2)
+    if proj.is_cuda:
+        assert proj.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_rotary_store(_p(proj), proj.stride(0), off_q, off_k, off_v, _p(inv_freq), _p(head_scale), _p(q_out),
+                                          _p(k_cache), _p(v_cache), _p(step.cu_q), _p(step.ctx_lens), _p(step.tok_seq),
+                                          _p(step.block_tables), step.block_tables.stride(0), T, H, G, D, Dv, rot_dims, page,
+                                          _DT[proj.dtype], _stream(proj)), "lv_rotary_store")
+        return q_out
+    pos = _positions(step, proj.device)
+    q = _rotate(proj[:, off_q:off_q + H * D].float().view(T, H, D), pos, inv_freq, rot_dims)
+    if head_scale is not None:
+        q = q * head_scale.view(1, H, 1)
+    q_out.copy_(q.reshape(T, H * D))
+    k = _rotate(proj[:, off_k:off_k + G * D].float().view(T, G, D), pos, inv_freq, rot_dims).reshape(T, G * D).to(k_cache.dtype)
+    v = proj[:, off_v:off_v + G * Dv]
+    kc, vc = k_cache.view(-1, G * D), v_cache.view(-1, G * Dv)
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        bt = step.host_block_tables[b]
+        for r in range(n):
+            sl = _token_slot(bt, ctx + r, page)
+            kc[sl] = k[q0 + r]
+            vc[sl] = v[q0 + r]
+        q0 += n
+    return q_out
 
 
 def latent_prep(proj, off_q, off_kv, q_w, kv_w, inv_freq, cache, step, Rq, R, Dr, rot_dims, eps):
@@ -478,11 +616,12 @@ def latent_out_gate(o, gate, per_channel: bool):
 
 
 # ------------------------------------------------------------------------------ mixture of experts
-def moe_route(logits, correction, top, groups=1, keep=1):
+def moe_route(logits, correction, top, groups=1, keep=1, normalize=True):
     """logits f32 [T, E] -> (ids int32 [T, top], weights f32 [T, top], dense f32 [T, E]).
     Scores s = sigmoid(logits); the choice goes by s + correction; with `groups` > 1 only experts of the
     `keep` blocks of consecutive experts ranked highest by the sum of their two top selection scores stay in the selection; weights are the
-    chosen s over their sum (+ 1e-20); dense holds them at the chosen experts and 0 elsewhere."""
+    chosen s over their sum (+ 1e-20), or the chosen s themselves without `normalize`; dense holds them at the
+    chosen experts and 0 elsewhere. correction may be None."""
     T, E = logits.shape
     _f32(logits, correction)
     dev = logits.device
@@ -492,7 +631,7 @@ def moe_route(logits, correction, top, groups=1, keep=1):
     if logits.is_cuda:
         lib = _mixlib.load()
         _mixlib.check(lib.lv_moe_route(_p(logits), _p(correction), _p(ids), _p(w), _p(dense), T, E, top, groups, keep,
-                                       _stream(logits)), "lv_moe_route")
+                                       int(normalize), _stream(logits)), "lv_moe_route")
         return ids, w, dense
     s = torch.sigmoid(logits)
     c = s + correction if correction is not None else s.clone()
@@ -504,7 +643,8 @@ def moe_route(logits, correction, top, groups=1, keep=1):
         c = cg.masked_fill(~kept[:, :, None], float("-inf")).reshape(T, E)
     idx = c.topk(top, -1).indices
     ws = s.gather(1, idx)
-    ws = ws / (ws.sum(-1, keepdim=True) + 1e-20)
+    if normalize:
+        ws = ws / (ws.sum(-1, keepdim=True) + 1e-20)
     ids.copy_(idx)
     w.copy_(ws)
     dense.zero_().scatter_(1, idx, ws)
@@ -556,6 +696,35 @@ def moe_grouped_ff(h, ids, weights, up_w, down_w, E, Fe):
     return out
 
 
+def moe_grouped_glu_ff(h, ids, weights, up_w, down_w, E, Fe, limit, alpha):
+    """y[t] = sum_k W_down,e glu(weights[t, k] * W_gu,e h[t]) with e = ids[t, k] and glu the clamped gated unit of
+    expert_glu: the choice's weight scales what the expert reads, the outputs are summed as they are. Computed
+    expert by expert on rows sorted by expert. up_w [E*2*Fe, W] (per expert gate rows, then up rows), down_w [W, E*Fe]
+    (a column block of a wider weight is fine: its row stride is passed on). Returns act [T, W]."""
+    T, W = h.shape
+    top = ids.size(1)
+    out = torch.empty(T, W, dtype=h.dtype, device=h.device)
+    if h.is_cuda:
+        assert moe_grouped_ok(h, Fe) and h.is_contiguous() and up_w.is_contiguous() and down_w.stride(1) == 1
+        assert down_w.stride(0) % 8 == 0 and down_w.data_ptr() % 16 == 0 and up_w.data_ptr() % 16 == 0
+        assert ids.dtype == torch.int32 and ids.is_contiguous() and weights.is_contiguous() and weights.dtype == torch.float32
+        lib = _mixlib.load()
+        ws = torch.empty(lib.lv_moe_grouped_workspace_bytes(T, W, Fe, E, top), dtype=torch.uint8, device=h.device)
+        _mixlib.check(lib.lv_moe_grouped_glu_ff(_p(h), _p(ids), _p(weights), _p(up_w), _p(down_w), down_w.stride(0), _p(out),
+                                                _p(ws), T, W, Fe, E, top, limit, alpha, _stream(h)), "lv_moe_grouped_glu_ff")
+        return out
+    acc = torch.zeros(T, W)
+    for e in range(E):
+        t_idx, k_idx = (ids == e).nonzero(as_tuple=True)
+        if t_idx.numel() == 0:
+            continue
+        pre = F.linear(h[t_idx], up_w[e * 2 * Fe:(e + 1) * 2 * Fe])
+        a = expert_glu(pre, 1, Fe, limit, alpha, in_scale=weights[t_idx, k_idx][:, None].contiguous())
+        acc.index_add_(0, t_idx, F.linear(a, down_w[:, e * Fe:(e + 1) * Fe]).float())
+    out.copy_(acc)
+    return out
+
+
 def moe_sort(ids, E, align=1):
     """ids int32 [T, top] -> (sorted_pair [M + E * align], inv [T, top], offsets [E + 1]), int32: the (token, choice)
     pairs in expert order, the row each pair got, and the first row of every expert. Every expert starts on a multiple
@@ -583,17 +752,20 @@ def moe_sort(ids, E, align=1):
     return sorted_pair, inv.view_as(ids), offsets.to(torch.int32)
 
 
-def moe_combine(rows, inv, weights):
-    """rows act [M, W] (expert outputs in sorted order) -> act [T, W] = sum_k weights[t, k] * rows[inv[t, k]], in f32."""
+def moe_combine(rows, inv, weights=None):
+    """rows act [M, W] (expert outputs in sorted order) -> act [T, W] = sum_k weights[t, k] * rows[inv[t, k]], in f32
+    (weights None: the plain sum)."""
     T, top = inv.shape
     W = rows.size(1)
     out = torch.empty(T, W, dtype=rows.dtype, device=rows.device)
     if rows.is_cuda:
-        assert rows.dtype == torch.bfloat16 and rows.is_contiguous() and W % 4 == 0 and weights.dtype == torch.float32
+        assert rows.dtype == torch.bfloat16 and rows.is_contiguous() and W % 4 == 0
+        assert weights is None or (weights.dtype == torch.float32 and weights.is_contiguous())
         lib = _mixlib.load()
         _mixlib.check(lib.lv_moe_combine(_p(rows), _p(inv), _p(weights), _p(out), T, W, top, _stream(rows)), "lv_moe_combine")
         return out
-    out.copy_((rows[inv.long()].float() * weights[:, :, None]).sum(1))
+    picked = rows[inv.long()].float()
+    out.copy_((picked * weights[:, :, None] if weights is not None else picked).sum(1))
     return out
 
 

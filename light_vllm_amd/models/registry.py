@@ -26,10 +26,16 @@ def _bokulorn():
     return BokulornForCausalLM
 
 
+def _givozen():
+    from .givozen import GivozenForCausalLM
+    return GivozenForCausalLM
+
+
 MODELS = {
     "Qwen3ForCausalLM": _qwen3,
     "Kagalorn": _kagalorn,
     "Bokulorn": _bokulorn,
+    "Givozen": _givozen,
 }
 DEFAULT = "Qwen3ForCausalLM"
 
