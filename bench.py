@@ -885,6 +885,163 @@ def bokulorn_leg(sizes, batch, prompt_len, new_tokens):
     print(json.dumps(out), flush=True)
 
 
+# --mixers-design givozen: the Givozen design (gated rotary attention with head temperatures, sublayers normed on
+# both sides, PolyNorm and gated-expert feed-forwards, a looped stretch of layers) beside Bokulorn, the closest existing
+# model (one f32 residual with offset norms, the same paged attention kernel without a window, a mixture of experts),
+# at equal width, layer runs, head counts and active feed-forward parameters.
+GIVOZEN_SIZES = {
+    "2k": dict(experts=32, top=4, expert_ff=768, shared_ff=1024, rot_dims=64),
+    "4k": dict(experts=32, top=4, expert_ff=1536, shared_ff=2048, rot_dims=64),
+}
+
+
+def _givozen_config(z, gz):
+    from light_vllm_amd.models.givozen import GivozenConfig
+    att = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+           "rot": {"base": 500000.0, "dims": gz["rot_dims"], "scaling": {"factor": 4.0, "low": 1.0, "high": 2.0, "original": 2048}}}
+    moe = {"kind": "moe", "expert": {"ff": gz["expert_ff"], "limit": 7.0}, "router": {"experts": gz["experts"], "top": gz["top"]},
+           "shared": {"ff": gz["shared_ff"], "limit": 7.0}}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    looped = 2 if z["layers"] >= 6 else 1      # layers that run twice: as many layer runs as the other model has layers
+    n = z["layers"] - looped
+    layers = [{"type": "attention", "mixer": att, "mlp": dense if i == 0 else moe} for i in range(n)]
+    return GivozenConfig.from_dict({"vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "layers": layers,
+                                    "loop": {"start": 1, "stop": 1 + looped, "times": 2}})
+
+
+def _givozen_kernel_table(z, gz, bz, dev, batch, prompt_len):
+    """Each kernel of the design alone at one layer's shapes (prompt step and decode step), beside the Bokulorn
+    (or Kagalorn) kernel that does the like job."""
+    from light_vllm_amd import mix_ops
+    from light_vllm_amd.layers.moe import GLUSparseMoE, SparseMoE
+    from light_vllm_amd.layers.rotary_attention import NO_WINDOW
+    from light_vllm_amd.utils.context import RaggedStep
+    bf = torch.bfloat16
+    W, H, G, D = z["width"], z["heads"], z["kv_heads"], z["dim"]
+    E, top, Fe, Fs, rd = gz["experts"], gz["top"], gz["expert_ff"], gz["shared_ff"], gz["rot_dims"]
+    R, Dr, Rq = bz["kv_rank"], bz["rot_dim"], bz["q_rank"]
+    page = 256
+    rows = []
+
+    def step_of(lens_q, ctx):
+        B = len(lens_q)
+        cu, tok = [0], []
+        for b, n_ in enumerate(lens_q):
+            cu.append(cu[-1] + n_)
+            tok += [b] * n_
+        per = -(-(max(ctx) + max(lens_q)) // page)
+        tables = [[b * per + j for j in range(per)] for b in range(B)]
+        i32 = dict(dtype=torch.int32, device=dev)
+        return RaggedStep(torch.tensor(cu, **i32), torch.tensor(ctx, **i32), torch.arange(B, **i32),
+                          torch.tensor(tok, **i32), torch.tensor(tables, **i32), lens_q, ctx, list(range(B)), tables), B * per
+
+    def add(name, phase, fn, nbytes=0, flops=0, like=None):
+        us = _event_time(fn, 20, 3) * 1e6
+        rec = {"kernel": name, "phase": phase, "us": round(us, 1)}
+        if nbytes:
+            rec["of_hbm_roofline"] = round(nbytes / us / 1e3 / (HBM_BPS / 1e9), 3)
+        if flops:
+            rec["TFLOPs"] = round(flops / us / 1e6, 2)
+            rec["of_mfma_roofline"] = round(flops / us / 1e6 / (MFMA_FLOPS / 1e12), 4)
+        if like:
+            rec["like"] = like
+        rows.append(rec)
+
+    old_default = torch.get_default_dtype()
+    torch.set_default_dtype(bf)
+    try:
+        moe = GLUSparseMoE(W, Fe, E, top, 7.0, 1.702, Fs, 7.0).to(dev)
+        bmoe = SparseMoE(W, z["ff"] // bz["top"], bz["experts"], bz["top"], bz["groups"], bz["keep"]).to(dev)
+    finally:
+        torch.set_default_dtype(old_default)
+    for prm in list(moe.parameters()) + list(bmoe.parameters()):
+        prm.data.normal_(0.0, 0.02)
+    for phase, lens_q, ctx in (("prompt", [prompt_len] * batch, [0] * batch), ("decode", [1] * batch, [prompt_len] * batch)):
+        step, pages = step_of(lens_q, ctx)
+        T = sum(lens_q)
+        x = torch.randn(T, W, device=dev)
+        y1, y2 = torch.randn(T, W, device=dev, dtype=bf), torch.randn(T, W, device=dev, dtype=bf)
+        nw = torch.zeros(W, device=dev)
+        add("sandwich_add_norm", phase, lambda: mix_ops.sandwich_add_norm(x, y1, nw, None, None, nw, 1.0, 1e-6, bf), nbytes=T * W * 12)
+        add("sandwich_add_norm (start of a pass)", phase, lambda: mix_ops.sandwich_add_norm(x, y1, nw, y2, nw, nw, 1.0, 1e-6, bf),
+            nbytes=T * W * 14)
+        add("bokulorn residual_add_norm", phase, lambda: mix_ops.residual_add_norm(x, y1, y2, nw, 1.0, 1e-6, bf), nbytes=T * W * 14,
+            like="sandwich_add_norm")
+        # attention: rotation + cache write, then the paged kernel
+        cols = H * D + 2 * G * D + H
+        proj = torch.randn(T, cols, device=dev, dtype=bf)
+        inv_freq = mix_ops.rotary_inv_freq(rd, 500000.0, dev)
+        temp = torch.ones(H, device=dev)
+        kc = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        vc = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        add("rotary_store", phase, lambda: mix_ops.rotary_store(proj, 0, H * D, H * D + G * D, inv_freq, temp, kc, vc, step, H, G, D, D, rd),
+            nbytes=T * (H * D + 2 * G * D) * 4)
+        lproj = torch.randn(T, Rq + R + Dr + H, device=dev, dtype=bf)
+        lcache = torch.zeros(pages, page, R + Dr, device=dev, dtype=bf)
+        qw, kw_ = torch.ones(Rq, device=dev), torch.ones(R, device=dev)
+        lfreq = mix_ops.rotary_inv_freq(Dr, 10000.0, dev)
+        add("bokulorn latent_prep", phase, lambda: mix_ops.latent_prep(lproj, 0, Rq, qw, kw_, lfreq, lcache, step, Rq, R, Dr, Dr, 1e-6),
+            nbytes=T * (Rq * 4 + (R + Dr) * 4), like="rotary_store")
+        q = mix_ops.rotary_store(proj, 0, H * D, H * D + G * D, inv_freq, temp, kc, vc, step, H, G, D, D, rd)
+        gate = proj[:, H * D + 2 * G * D:]
+        keys = sum(i + 1 for n_, c0 in zip(lens_q, ctx) for i in range(c0, c0 + n_))
+        attn = lambda: mix_ops.window_pool_attention(q, kc, vc, None, None, gate, step, H, G, D, D, NO_WINDOW, 0, D ** -0.5,  # noqa: E731
+                                                     has_sink=False, gate_per_head=True)
+        q_abs = torch.randn(T, H * (R + Dr), device=dev, dtype=bf)
+        lc = lcache.unsqueeze(2)
+        lattn = lambda: mix_ops.window_pool_attention(q_abs, lc, lc[..., :R], None, None, None, step, H, 1, R + Dr, R,  # noqa: E731
+                                                      NO_WINDOW, 0, 0.07, has_sink=False)
+        if phase == "prompt":
+            add("gated rotary attention", phase, attn, flops=keys * H * D * 4)
+            add("bokulorn latent attention", phase, lattn, flops=keys * H * (2 * R + Dr) * 2, like="gated rotary attention")
+        else:
+            add("gated rotary attention", phase, attn, nbytes=keys * G * D * 4)
+            add("bokulorn latent attention", phase, lattn, nbytes=keys * (R + Dr) * 2, like="gated rotary attention")
+        # feed-forwards
+        h = torch.randn(T, W, device=dev, dtype=bf)
+        zf = torch.randn(T, z["ff"], device=dev, dtype=bf)
+        coef = torch.tensor([0.6, 0.3, 0.1, 0.0], device=dev)
+        add("polynorm", phase, lambda: mix_ops.polynorm(zf, coef, 1e-6), nbytes=T * z["ff"] * 4)
+        zg = torch.randn(T, 2 * z["ff"], device=dev, dtype=bf)
+        add("kagalorn clamped_glu", phase, lambda: mix_ops.clamped_glu(zg, 7.0, 1.702), nbytes=T * z["ff"] * 6, like="polynorm")
+        with torch.inference_mode():
+            wu = torch.randn(z["ff"], W, device=dev, dtype=bf) * 0.02
+            wd = torch.randn(W, z["ff"], device=dev, dtype=bf) * 0.02
+            add("dense PolyNorm feed-forward", phase,
+                lambda: torch.nn.functional.linear(mix_ops.polynorm(torch.nn.functional.linear(h, wu), coef, 1e-6), wd),
+                flops=T * z["ff"] * W * 4)
+            wg = torch.randn(2 * z["ff"], W, device=dev, dtype=bf) * 0.02
+            add("kagalorn dense feed-forward", phase,
+                lambda: torch.nn.functional.linear(mix_ops.clamped_glu(torch.nn.functional.linear(h, wg), 7.0, 1.702), wd),
+                flops=T * z["ff"] * W * 6, like="dense PolyNorm feed-forward")
+            weight_bytes = (min(T * top, E) * 3 * Fe + 3 * Fs) * W * 2
+            bweight_bytes = min(T * bz["top"], bz["experts"]) * 2 * (z["ff"] // bz["top"]) * W * 2
+            add("gated-expert feed-forward (router to sum, shared expert)", phase, lambda: moe(h),
+                flops=T * (top * Fe + Fs) * W * 6, nbytes=weight_bytes if phase == "decode" else 0)
+            add("bokulorn moe feed-forward", phase, lambda: bmoe(h), flops=T * bz["top"] * (z["ff"] // bz["top"]) * W * 4,
+                nbytes=bweight_bytes if phase == "decode" else 0, like="gated-expert feed-forward (router to sum, shared expert)")
+    return rows
+
+
+def givozen_leg(sizes, batch, prompt_len, new_tokens):
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    out = {"metric": "mixers: Givozen beside Bokulorn at equal size", "dtype": "bf16", "data": "synthetic, random weights",
+           "batch": batch, "prompt_len": prompt_len, "new_tokens": new_tokens, "sizes": []}
+    for name in sizes:
+        z, gz, bz = MIXER_SIZES[name], GIVOZEN_SIZES[name], BOKULORN_SIZES[name]
+        rec = {"size": name, **z, **gz}
+        cache_tokens = batch * 256 * (-(-(prompt_len + new_tokens) // 256))
+        kw = dict(kvcache_block_size=256, max_cache_tokens=cache_tokens)
+        rec["givozen"] = _engine_rates(_givozen_config(z, gz), batch, prompt_len, new_tokens, **kw)
+        rec["givozen_graph"] = _engine_rates(_givozen_config(z, gz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        rec["bokulorn"] = _engine_rates(_bokulorn_config(z, bz), batch, prompt_len, new_tokens, **kw)
+        rec["bokulorn_graph"] = _engine_rates(_bokulorn_config(z, bz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        rec["kernels"] = _givozen_kernel_table(z, gz, bz, dev, batch, prompt_len)
+        out["sizes"].append(rec)
+    print(json.dumps(out), flush=True)
+
+
 def mixers_leg(sizes, batch, prompt_len, new_tokens):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -956,12 +1113,15 @@ def main():
                          "(proves launcher, rendezvous, graph and JSON path; not a measurement)")
     ap.add_argument("--mixers", default="", help="comma list of sizes (2k, 4k): instead of the default workload, "
                     "run the Kagalorn design beside Qwen3 at equal size and time its kernels one by one")
-    ap.add_argument("--mixers-design", default="kagalorn", choices=("kagalorn", "bokulorn"),
-                    help="with --mixers: kagalorn (beside Qwen3) or bokulorn (beside Kagalorn, its closest relative)")
+    ap.add_argument("--mixers-design", default="kagalorn", choices=("kagalorn", "bokulorn", "givozen"),
+                    help="with --mixers: kagalorn (beside Qwen3), bokulorn (beside Kagalorn, its closest relative) or "
+                         "givozen (beside Bokulorn, its closest relative)")
     ap.add_argument("--mixers-batch", type=int, default=16)
     ap.add_argument("--mixers-prompt", type=int, default=1024)
     ap.add_argument("--mixers-new", type=int, default=17)
     args = ap.parse_args()
+    if args.mixers and args.mixers_design == "givozen":
+        return givozen_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
     if args.mixers and args.mixers_design == "bokulorn":
         return bokulorn_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
     if args.mixers:
