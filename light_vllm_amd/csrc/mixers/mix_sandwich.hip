@@ -23,7 +23,7 @@ __device__ __forceinline__ float block_sum4(float v, float* red) {
   return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void sandwich_add_norm_kernel(float* __restrict__ x, const T* __restrict__ y,
                                                                  const float* __restrict__ post_w, const T* __restrict__ rows,
                                                                  const float* __restrict__ vec, const float* __restrict__ w,
@@ -32,33 +32,68 @@ __global__ __launch_bounds__(256) void sandwich_add_norm_kernel(float* __restric
   float* red = lds + W;
   const int64_t t = blockIdx.x;
   float* xt = x + t * W;
+  const int first = threadIdx.x * VEC, stride = blockDim.x * VEC;      // VEC = 4 when W % 4 == 0 and all rows are aligned
   float inv_y = 0.0f;
   if (y != nullptr) {
     float ss = 0.0f;
-    for (int i = threadIdx.x; i < W; i += blockDim.x) {
-      const float v = ldf(y + t * W + i);
-      lds[i] = v;
-      ss += v * v;
+    for (int i = first; i < W; i += stride) {
+      if constexpr (VEC == 4) {
+        const float4 v = ld4(y + t * W + i);
+        st4(lds + i, v);
+        ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+      } else {
+        const float v = ldf(y + t * W + i);
+        lds[i] = v;
+        ss += v * v;
+      }
     }
     inv_y = 1.0f / sqrtf(block_sum4(ss, red) / static_cast<float>(W) + eps);
   }
   float ss = 0.0f;
   const bool changes = y != nullptr || rows != nullptr || vec != nullptr;
-  for (int i = threadIdx.x; i < W; i += blockDim.x) {                  // every thread reads back its own entries of lds
-    float v = xt[i];
-    if (y != nullptr) v += lds[i] * inv_y * (w_offset + post_w[i]);
-    if (rows != nullptr) v += ldf(rows + t * W + i);
-    if (vec != nullptr) v += vec[i];
-    if (changes) xt[i] = v;
-    lds[i] = v;
-    ss += v * v;
+  for (int i = first; i < W; i += stride) {                            // every thread reads back its own entries of lds
+    if constexpr (VEC == 4) {
+      float4 v = ld4(xt + i);
+      if (y != nullptr) {
+        const float4 a = ld4(lds + i), g = ld4(post_w + i);
+        v.x += a.x * inv_y * (w_offset + g.x); v.y += a.y * inv_y * (w_offset + g.y);
+        v.z += a.z * inv_y * (w_offset + g.z); v.w += a.w * inv_y * (w_offset + g.w);
+      }
+      if (rows != nullptr) {
+        const float4 a = ld4(rows + t * W + i);
+        v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+      }
+      if (vec != nullptr) {
+        const float4 a = ld4(vec + i);
+        v.x += a.x; v.y += a.y; v.z += a.z; v.w += a.w;
+      }
+      if (changes) st4(xt + i, v);
+      st4(lds + i, v);
+      ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+    } else {
+      float v = xt[i];
+      if (y != nullptr) v += lds[i] * inv_y * (w_offset + post_w[i]);
+      if (rows != nullptr) v += ldf(rows + t * W + i);
+      if (vec != nullptr) v += vec[i];
+      if (changes) xt[i] = v;
+      lds[i] = v;
+      ss += v * v;
+    }
   }
   if (out == nullptr) return;
   const float inv = 1.0f / sqrtf(block_sum4(ss, red) / static_cast<float>(W) + eps);
-  for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + t * W + i, lds[i] * inv * (w_offset + w[i]));
+  for (int i = first; i < W; i += stride) {
+    if constexpr (VEC == 4) {
+      const float4 v = ld4(lds + i), g = ld4(w + i);
+      st4(out + t * W + i, float4{v.x * inv * (w_offset + g.x), v.y * inv * (w_offset + g.y), v.z * inv * (w_offset + g.z),
+                                  v.w * inv * (w_offset + g.w)});
+    } else {
+      stf(out + t * W + i, lds[i] * inv * (w_offset + w[i]));
+    }
+  }
 }
 
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void rotary_store_kernel(const T* __restrict__ proj, int64_t ld, int off_q, int off_k,
                                                            int off_v, const float* __restrict__ inv_freq,
                                                            const float* __restrict__ head_scale, T* __restrict__ q_out,
@@ -68,7 +103,7 @@ __global__ __launch_bounds__(256) void rotary_store_kernel(const T* __restrict__
                                                            const int32_t* __restrict__ tok_seq,
                                                            const int32_t* __restrict__ block_tables, int bt_stride, int H,
                                                            int G, int D, int Dv, int rot_dims, int page) {
-  extern __shared__ float cs[];                      // [rot_dims/2] cosines | [rot_dims/2] sines
+  extern __shared__ __attribute__((aligned(16))) float cs[];   // [rot_dims/2] cosines | [rot_dims/2] sines
   const int64_t t = blockIdx.x;
   const int b = tok_seq[t];
   const int pos = ctx_lens[b] + static_cast<int>(t) - cu_q[b];
@@ -83,12 +118,40 @@ __global__ __launch_bounds__(256) void rotary_store_kernel(const T* __restrict__
   }
   __syncthreads();
   const T* row = proj + t * ld;
+  const int HD = H * D, GD = G * D, GDv = G * Dv;
+  if constexpr (VEC == 4) {
+    // four consecutive entries of a head lie wholly in its first rotated half, its second, or its unrotated rest
+    auto turned4 = [&](const T* head, int j) -> float4 {
+      const float4 v = ld4(head + j);
+      if (j >= rot_dims) return v;
+      if (j < half) {
+        const float4 u = ld4(head + j + half), c = ld4(cs + j), sn = ld4(cs + half + j);
+        return float4{v.x * c.x - u.x * sn.x, v.y * c.y - u.y * sn.y, v.z * c.z - u.z * sn.z, v.w * c.w - u.w * sn.w};
+      }
+      const float4 u = ld4(head + j - half), c = ld4(cs + j - half), sn = ld4(cs + j);
+      return float4{v.x * c.x + u.x * sn.x, v.y * c.y + u.y * sn.y, v.z * c.z + u.z * sn.z, v.w * c.w + u.w * sn.w};
+    };
+    for (int i = threadIdx.x * 4; i < HD; i += blockDim.x * 4) {
+      const int h = i / D, j = i - h * D;
+      float4 v = turned4(row + off_q + h * D, j);
+      if (head_scale != nullptr) {
+        const float f = head_scale[h];
+        v.x *= f; v.y *= f; v.z *= f; v.w *= f;
+      }
+      st4(q_out + t * HD + i, v);
+    }
+    for (int i = threadIdx.x * 4; i < GD; i += blockDim.x * 4) {
+      const int g = i / D, j = i - g * D;
+      st4(k_cache + slot * GD + i, turned4(row + off_k + g * D, j));
+    }
+    for (int i = threadIdx.x * 4; i < GDv; i += blockDim.x * 4) st4(v_cache + slot * GDv + i, ld4(row + off_v + i));
+    return;
+  }
   auto turned = [&](const T* head, int j) -> float {
     if (j >= rot_dims) return ldf(head + j);
     if (j < half) return ldf(head + j) * cs[j] - ldf(head + j + half) * cs[half + j];
     return ldf(head + j) * cs[j - half] + ldf(head + j - half) * cs[j];     // cs[half + (j - half)]
   };
-  const int HD = H * D, GD = G * D, GDv = G * Dv;
   for (int i = threadIdx.x; i < HD; i += blockDim.x) {
     const int h = i / D, j = i - h * D;
     const float v = turned(row + off_q + h * D, j);
@@ -101,18 +164,27 @@ __global__ __launch_bounds__(256) void rotary_store_kernel(const T* __restrict__
   for (int i = threadIdx.x; i < GDv; i += blockDim.x) v_cache[slot * GDv + i] = row[off_v + i];
 }
 
-template <typename T>
+template <typename T, int VEC>
 __global__ __launch_bounds__(256) void polynorm_kernel(const T* __restrict__ in, int64_t ld_in, const float* __restrict__ coef,
                                                        T* __restrict__ out, int F, float eps) {
   __shared__ float red[3][4];
   const int64_t t = blockIdx.x;
   const T* z = in + t * ld_in;
+  const int first = threadIdx.x * VEC, stride = blockDim.x * VEC;      // VEC = 4 when F and ld_in are multiples of 4 and the rows aligned
   float s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
-  for (int i = threadIdx.x; i < F; i += blockDim.x) {
-    const float v = ldf(z + i), v2 = v * v;
+  auto take = [&](float v) {
+    const float v2 = v * v;
     s1 += v2;
     s2 += v2 * v2;
     s3 += v2 * v2 * v2;
+  };
+  for (int i = first; i < F; i += stride) {
+    if constexpr (VEC == 4) {
+      const float4 v = ld4(z + i);
+      take(v.x); take(v.y); take(v.z); take(v.w);
+    } else {
+      take(ldf(z + i));
+    }
   }
   s1 = wave_sum(s1);
   s2 = wave_sum(s2);
@@ -129,9 +201,14 @@ __global__ __launch_bounds__(256) void polynorm_kernel(const T* __restrict__ in,
   const float b = coef[1] / sqrtf(((red[1][0] + red[1][1]) + (red[1][2] + red[1][3])) / n + eps);
   const float c = coef[2] / sqrtf(((red[2][0] + red[2][1]) + (red[2][2] + red[2][3])) / n + eps);
   const float e = coef[3];
-  for (int i = threadIdx.x; i < F; i += blockDim.x) {
-    const float v = ldf(z + i);
-    stf(out + t * F + i, ((c * v + b) * v + a) * v + e);
+  auto poly = [&](float v) { return ((c * v + b) * v + a) * v + e; };
+  for (int i = first; i < F; i += stride) {                            // the row again: it is still in the cache
+    if constexpr (VEC == 4) {
+      const float4 v = ld4(z + i);
+      st4(out + t * F + i, float4{poly(v.x), poly(v.y), poly(v.z), poly(v.w)});
+    } else {
+      stf(out + t * F + i, poly(ldf(z + i)));
+    }
   }
 }
 
@@ -172,18 +249,21 @@ int lv_sandwich_add_norm(void* x, const void* y, const void* post_w, const void*
   const size_t shm = static_cast<size_t>(W + 4) * sizeof(float);
   if (shm > 64 * 1024) return fail(-2, "lv_sandwich_add_norm: width %d too large", W);
   dim3 grid(static_cast<unsigned>(T)), block(256);
-  if (dtype == LV_MIX_BF16)
-    sandwich_add_norm_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<float*>(x), static_cast<const bf16_t*>(y), static_cast<const float*>(post_w),
-        static_cast<const bf16_t*>(rows), static_cast<const float*>(vec), static_cast<const float*>(w), w_offset,
-        static_cast<bf16_t*>(out), W, eps);
-  else if (dtype == LV_MIX_F32)
-    sandwich_add_norm_kernel<float><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<float*>(x), static_cast<const float*>(y), static_cast<const float*>(post_w),
-        static_cast<const float*>(rows), static_cast<const float*>(vec), static_cast<const float*>(w), w_offset,
-        static_cast<float*>(out), W, eps);
-  else
+  auto aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec4 = W % 4 == 0 && aligned(x) && aligned(y) && aligned(post_w) && aligned(rows) && aligned(vec) && aligned(w) &&
+                    aligned(out);
+#define LVMIX_SANDWICH(TT, VV)                                                                                  \
+  sandwich_add_norm_kernel<TT, VV><<<grid, block, shm, as_stream(stream)>>>(                                   \
+      static_cast<float*>(x), static_cast<const TT*>(y), static_cast<const float*>(post_w), static_cast<const TT*>(rows), \
+      static_cast<const float*>(vec), static_cast<const float*>(w), w_offset, static_cast<TT*>(out), W, eps)
+  if (dtype == LV_MIX_BF16) {
+    if (vec4) LVMIX_SANDWICH(bf16_t, 4); else LVMIX_SANDWICH(bf16_t, 1);
+  } else if (dtype == LV_MIX_F32) {
+    if (vec4) LVMIX_SANDWICH(float, 4); else LVMIX_SANDWICH(float, 1);
+  } else {
     return fail(-1, "lv_sandwich_add_norm: dtype %d", dtype);
+  }
+#undef LVMIX_SANDWICH
   return launched("lv_sandwich_add_norm");
 }
 
@@ -199,20 +279,25 @@ int lv_rotary_store(const void* proj, int64_t ld, int off_q, int off_k, int off_
       off_q + static_cast<int64_t>(H) * D > ld || off_k + static_cast<int64_t>(G) * D > ld ||
       off_v + static_cast<int64_t>(G) * Dv > ld)
     return fail(-1, "lv_rotary_store: bad sizes");
-  const size_t shm = sizeof(float) * static_cast<size_t>(rot_dims > 0 ? rot_dims : 1);
+  const size_t shm = sizeof(float) * static_cast<size_t>(rot_dims > 0 ? rot_dims : 4);
   dim3 grid(static_cast<unsigned>(T)), block(256);
-  if (dtype == LV_MIX_BF16)
-    rotary_store_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<const bf16_t*>(proj), ld, off_q, off_k, off_v, static_cast<const float*>(inv_freq),
-        static_cast<const float*>(head_scale), static_cast<bf16_t*>(q_out), static_cast<bf16_t*>(k_cache),
-        static_cast<bf16_t*>(v_cache), cu_q, ctx_lens, tok_seq, block_tables, bt_stride, H, G, D, Dv, rot_dims, page);
-  else if (dtype == LV_MIX_F32)
-    rotary_store_kernel<float><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<const float*>(proj), ld, off_q, off_k, off_v, static_cast<const float*>(inv_freq),
-        static_cast<const float*>(head_scale), static_cast<float*>(q_out), static_cast<float*>(k_cache),
-        static_cast<float*>(v_cache), cu_q, ctx_lens, tok_seq, block_tables, bt_stride, H, G, D, Dv, rot_dims, page);
-  else
+  auto aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  // groups of four: head sizes, both halves of the rotated part and every column offset in multiples of 4
+  const bool vec4 = D % 4 == 0 && Dv % 4 == 0 && rot_dims % 8 == 0 && ld % 4 == 0 && off_q % 4 == 0 && off_k % 4 == 0 &&
+                    off_v % 4 == 0 && aligned(proj) && aligned(q_out) && aligned(k_cache) && aligned(v_cache);
+#define LVMIX_ROTARY(TT, VV)                                                                                          \
+  rotary_store_kernel<TT, VV><<<grid, block, shm, as_stream(stream)>>>(                                               \
+      static_cast<const TT*>(proj), ld, off_q, off_k, off_v, static_cast<const float*>(inv_freq),                     \
+      static_cast<const float*>(head_scale), static_cast<TT*>(q_out), static_cast<TT*>(k_cache), static_cast<TT*>(v_cache), \
+      cu_q, ctx_lens, tok_seq, block_tables, bt_stride, H, G, D, Dv, rot_dims, page)
+  if (dtype == LV_MIX_BF16) {
+    if (vec4) LVMIX_ROTARY(bf16_t, 4); else LVMIX_ROTARY(bf16_t, 1);
+  } else if (dtype == LV_MIX_F32) {
+    if (vec4) LVMIX_ROTARY(float, 4); else LVMIX_ROTARY(float, 1);
+  } else {
     return fail(-1, "lv_rotary_store: dtype %d", dtype);
+  }
+#undef LVMIX_ROTARY
   return launched("lv_rotary_store");
 }
 
@@ -221,14 +306,19 @@ int lv_polynorm(const void* in, int64_t ld_in, const void* coef, void* out, int6
   if (T == 0) return 0;
   if (!in || !coef || !out || T < 0 || F <= 0 || ld_in < F) return fail(-1, "lv_polynorm: bad arguments");
   dim3 grid(static_cast<unsigned>(T)), block(256);
-  if (dtype == LV_MIX_BF16)
-    polynorm_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(static_cast<const bf16_t*>(in), ld_in,
-                                                                 static_cast<const float*>(coef), static_cast<bf16_t*>(out), F, eps);
-  else if (dtype == LV_MIX_F32)
-    polynorm_kernel<float><<<grid, block, 0, as_stream(stream)>>>(static_cast<const float*>(in), ld_in,
-                                                                static_cast<const float*>(coef), static_cast<float*>(out), F, eps);
-  else
+  const bool vec4 = F % 4 == 0 && ld_in % 4 == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+#define LVMIX_POLY(TT, VV)                                                                                   \
+  polynorm_kernel<TT, VV><<<grid, block, 0, as_stream(stream)>>>(static_cast<const TT*>(in), ld_in,          \
+                                                                 static_cast<const float*>(coef), static_cast<TT*>(out), F, eps)
+  if (dtype == LV_MIX_BF16) {
+    if (vec4) LVMIX_POLY(bf16_t, 4); else LVMIX_POLY(bf16_t, 1);
+  } else if (dtype == LV_MIX_F32) {
+    if (vec4) LVMIX_POLY(float, 4); else LVMIX_POLY(float, 1);
+  } else {
     return fail(-1, "lv_polynorm: dtype %d", dtype);
+  }
+#undef LVMIX_POLY
   return launched("lv_polynorm");
 }
 

@@ -126,19 +126,6 @@ static int hc_launch(void* x, const void* y, const void* mix, const void* out_w,
 // ------------------------------------------------------------------------------------------------
 // x f32 [T, W] += y1 + y2 (either may be absent); out = x / sqrt(mean(x^2) + eps) * (w_offset + w).
 // Four elements per thread and access (16-byte loads of the residual, 8-byte loads of bf16 rows) when W is a multiple of 4.
-__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
-__device__ __forceinline__ float4 ld4(const bf16_t* p) {
-  const uint2 v = *reinterpret_cast<const uint2*>(p);
-  return float4{__builtin_bit_cast(float, v.x << 16), __builtin_bit_cast(float, v.x & 0xffff0000u),
-                __builtin_bit_cast(float, v.y << 16), __builtin_bit_cast(float, v.y & 0xffff0000u)};
-}
-__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
-__device__ __forceinline__ void st4(bf16_t* p, float4 v) {
-  bf16_t a, b, c, d;
-  stf(&a, v.x); stf(&b, v.y); stf(&c, v.z); stf(&d, v.w);
-  *reinterpret_cast<uint2*>(p) = uint2{static_cast<uint32_t>(a.bits) | (static_cast<uint32_t>(b.bits) << 16),
-                                       static_cast<uint32_t>(c.bits) | (static_cast<uint32_t>(d.bits) << 16)};
-}
 
 template <typename T, int VEC>
 __global__ __launch_bounds__(256) void residual_add_norm_kernel(float* __restrict__ x, const T* __restrict__ y1,

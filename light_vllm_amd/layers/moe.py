@@ -29,9 +29,10 @@ or groups whose weights are the chosen scores themselves, the weight applied to 
 and an optional shared expert of the same form that every token uses, times sigmoid(w_sg . h). Because the
 projections are linear, s * h enters as a factor on the pre-activations (mix_ops.expert_glu), and the shared
 expert's token gate as a factor on its activations, so all of it is GEMMs on h plus one elementwise kernel.
-Forms: masked (everything in one up GEMM and one down GEMM; any dtype and size) and gathered (bf16: sort, two
+Forms: masked (everything in one up GEMM and one down GEMM; any dtype and size), gathered (bf16: sort, two
 grouped GEMMs on the matrix cores with the gated unit in the first one's epilogue, sum; the shared expert as
-vendor GEMMs beside it).
+vendor GEMMs beside it) and sorted (bf16, eager steps with at least SORTED_FROM rows per expert: the same sort, then
+every expert's products as vendor GEMMs on its slice of the sorted rows).
 """
 from __future__ import annotations
 
@@ -112,17 +113,22 @@ class GLUSparseMoE(nn.Module):
         return mix_ops.moe_route(logits, None, self.top, 1, 1, normalize=False)
 
     def form(self, h: torch.Tensor) -> str:
-        if MOE_KERNEL in ("masked", "gathered"):
+        if MOE_KERNEL != "auto":
             return MOE_KERNEL
         ok = mix_ops.moe_grouped_ok(h, self.ff) and (self.E * self.ff + self.Fs) % 8 == 0
-        return "gathered" if ok and self.E >= GATHER_FROM * self.top else "masked"
+        if not (ok and self.E >= GATHER_FROM * self.top):
+            return "masked"
+        step = get_context().ragged
+        captured = step is not None and step.static
+        return "sorted" if not captured and h.size(0) * self.top >= SORTED_FROM * self.E else "gathered"
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         ids, weights, dense = self.route(h)
         E, Fe, Fs, T = self.E, self.ff, self.Fs, h.size(0)
-        if self.form(h) == "gathered":
-            routed_down = self.down_weight[:, :E * Fe]
-            y = mix_ops.moe_grouped_glu_ff(h, ids, weights, self.up_weight[:E * 2 * Fe], routed_down, E, Fe, self.limit, self.alpha)
+        form = self.form(h)
+        if form in ("gathered", "sorted"):
+            routed = mix_ops.moe_grouped_glu_ff if form == "gathered" else mix_ops.moe_sorted_glu_ff
+            y = routed(h, ids, weights, self.up_weight[:E * 2 * Fe], self.down_weight[:, :E * Fe], E, Fe, self.limit, self.alpha)
             if Fs:
                 up = F.linear(h, self.up_weight[E * 2 * Fe:])
                 a = mix_ops.expert_glu(up[:, :2 * Fs], 1, Fs, self.shared_limit, self.alpha, out_gate=up[:, 2 * Fs])

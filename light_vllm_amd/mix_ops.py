@@ -793,3 +793,27 @@ def moe_sorted_ff(h, ids, weights, up_w, down_w, E, Fe):
         if off[e + 1] > off[e]:
             torch.mm(act[off[e]:off[e + 1]], down_w[:, e * Fe:(e + 1) * Fe].t(), out=rows[off[e]:off[e + 1]])
     return moe_combine(rows, inv, weights)
+
+
+def moe_sorted_glu_ff(h, ids, weights, up_w, down_w, E, Fe, limit, alpha):
+    """The same sum as moe_grouped_glu_ff for large eager steps, the way moe_sorted_ff does it: rows sorted by expert on
+    the device, the experts' row counts read back once, each expert's gate|up product and down product as vendor GEMMs on
+    its slice of the sorted rows (slices padded to SORTED_ALIGN rows), the gated unit over all sorted rows in one launch
+    with every row's routing weight as the factor on its pre-activations, and the plain sum of every token's rows."""
+    T, W = h.shape
+    top = ids.size(1)
+    sorted_pair, inv, offsets = moe_sort(ids, E, SORTED_ALIGN)
+    off = offsets.tolist()
+    pairs = sorted_pair[:off[E]]
+    xs = h.index_select(0, torch.div(pairs, top, rounding_mode="floor"))
+    scale = weights.reshape(-1).index_select(0, pairs).unsqueeze(1).contiguous()
+    pre = torch.empty(off[E], 2 * Fe, dtype=h.dtype, device=h.device)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            torch.mm(xs[off[e]:off[e + 1]], up_w[e * 2 * Fe:(e + 1) * 2 * Fe].t(), out=pre[off[e]:off[e + 1]])
+    act = expert_glu(pre, 1, Fe, limit, alpha, in_scale=scale)
+    rows = torch.empty(off[E], W, dtype=h.dtype, device=h.device)
+    for e in range(E):
+        if off[e + 1] > off[e]:
+            torch.mm(act[off[e]:off[e + 1]], down_w[:, e * Fe:(e + 1) * Fe].t(), out=rows[off[e]:off[e + 1]])
+    return moe_combine(rows, inv, None)

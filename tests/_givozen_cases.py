@@ -67,8 +67,12 @@ def case_rotary_store(device, dtype):
     the head factor on queries only, keys and values in the cache rows the page table names."""
     from light_vllm_amd import mix_ops
     g = torch.Generator().manual_seed(2)
-    for (H, G, D, Dv, rot) in ((4, 2, 12, 10, K.ROT_A), (1, 1, 40, 70, {"base": 300.0, "dims": 40}), (5, 1, 6, 4, None),
-                               (6, 3, 16, 32, {"base": 10.0, "dims": 2}), (2, 2, 48, 16, {"base": 1e5, "dims": 32})):
+    shapes = ((4, 2, 12, 10, K.ROT_A, 0), (1, 1, 40, 70, {"base": 300.0, "dims": 40}, 0), (5, 1, 6, 4, None, 0),
+              (6, 3, 16, 32, {"base": 10.0, "dims": 2}, 0), (2, 2, 48, 16, {"base": 1e5, "dims": 32}, 0),
+              # columns and sizes in multiples of four: the kernel's four-at-a-time form, part of a head rotated, all of it, none
+              (2, 2, 48, 16, {"base": 1e5, "dims": 32}, 1), (3, 1, 8, 8, {"base": 40.0, "dims": 8}, 1), (2, 1, 16, 4, None, 1),
+              (4, 2, 64, 32, {"base": 2000.0, "dims": 24, "scaling": {"factor": 5.0, "low": 1.0, "high": 3.0, "original": 128}}, 1))
+    for (H, G, D, Dv, rot, lined_up) in shapes:
         for ctx in (29, 70000):
             page, T = 16, 21
             first = ctx // page
@@ -78,6 +82,8 @@ def case_rotary_store(device, dtype):
                 row[j] = p
             ld = 5 + H * D + G * D + G * Dv + 3
             off_q, off_k, off_v = 2, 2 + H * D + 1, 2 + H * D + 1 + G * D + 2
+            if lined_up:
+                ld, off_q, off_k, off_v = H * D + G * D + G * Dv + 4, 0, H * D, H * D + G * D
             proj = torch.randn(T, ld, generator=g).to(_dt(dtype))
             temp = 1 + 0.5 * torch.randn(H, generator=g)
             dims = int(rot["dims"]) if rot else 0
@@ -173,9 +179,10 @@ def case_polynorm(device, dtype):
         buf = (spread * torch.randn(T, Fd + 7, generator=g)).to(_dt(dtype))
         z = buf[:, 3:3 + Fd]
         coef = torch.tensor([0.7, 0.4, -0.2, 0.1]) + 0.1 * torch.randn(4, generator=g)
-        got = mix_ops.polynorm(z.to(device) if device == "cpu" else buf.to(device)[:, 3:3 + Fd], coef.to(device), 1e-5).cpu().to(F64)
         want = oracle.polynorm(z.to(F64), coef.to(F64), 1e-5)
-        assert torch.allclose(got, want, rtol=tol, atol=tol * want.abs().max().item()), (T, Fd, spread)
+        for zd in (buf.to(device)[:, 3:3 + Fd], z.contiguous().to(device)):          # a view of wider rows, and rows of their own
+            got = mix_ops.polynorm(zd, coef.to(device), 1e-5).cpu().to(F64)
+            assert torch.allclose(got, want, rtol=tol, atol=tol * want.abs().max().item()), (T, Fd, spread)
     # the three norms are separate: a row with one large entry has R(z^3) close to a one-hot vector
     z = torch.full((1, 64), 0.1); z[0, 5] = 20.0
     got = mix_ops.polynorm(z.to(_dt(dtype)).to(device), torch.tensor([0.0, 0.0, 1.0, 0.0], device=device), 1e-6).cpu().float()
@@ -211,8 +218,8 @@ def case_moe_ff(device, dtype):
     cases = [(48, 20, 6, 2, 12, 37), (40, 8, 3, 3, 0, 9), (64, 32, 8, 3, 48, 50), (64, 64, 4, 1, 0, 300), (32, 32, 5, 2, 24, 1),
              (96, 32, 16, 4, 8, 700)]
     for (W, Fe, E, top, Fs, T) in cases:
-        forms = ["masked"] + (["gathered"] if dtype == "bfloat16" and device != "cpu" and W % 32 == 0 and Fe % 32 == 0
-                              and (E * Fe + Fs) % 8 == 0 else []) + (["gathered"] if device == "cpu" else [])
+        forms = ["masked"] + (["gathered", "sorted"] if device == "cpu" or (dtype == "bfloat16" and W % 32 == 0 and Fe % 32 == 0
+                                                               and (E * Fe + Fs) % 8 == 0) else [])
         mlp = {"expert": {"ff": Fe, "limit": 0.6}, "router": {"experts": E, "top": top}}
         weights = {"router": 2 * torch.randn(E, W, generator=g) / W ** 0.5}
         for e in range(E):
