@@ -47,7 +47,7 @@ def test_engine_other_sizes(tmp_path, name):
     C.case_engine_schedules(DEV, "float32", tmp_path, cfg=getattr(K, name), seed=9)
 
 
-@pytest.mark.parametrize("seed", [101, 102])
+@pytest.mark.parametrize("seed", [102, 107])
 def test_engine_random_configs(tmp_path, seed):
     C.case_engine_random_config(DEV, "float32", tmp_path, seed)
 

@@ -58,7 +58,7 @@ def test_engine_other_sizes(gpu, tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("seed", [101, 102, 103, 104, 105, 106])
+@pytest.mark.parametrize("seed", [102, 104, 106, 107, 109, 110])
 def test_engine_random_configs(gpu, tmp_path, seed, dtype):
     C.case_engine_random_config(DEV, dtype, tmp_path, seed)
 
