@@ -131,16 +131,18 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
   }
 }
 
-// The choice of one token (one wave): z = its E router logits (global memory, or LDS written by this wave).
-__device__ __forceinline__ void route_token(const float* z, const float* __restrict__ correction, int32_t* __restrict__ ids,
-                                            float* __restrict__ weights, float* __restrict__ dense, int64_t t, int E, int top,
-                                            int groups, int keep, int normalize, float* rl) {
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
+                                                        int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                        float* __restrict__ dense, int E, int top, int groups, int keep,
+                                                        int normalize) {
+  extern __shared__ float rl[];
   float* s_lds = rl;              // [E] scores
   float* c_lds = rl + E;          // [E] selection scores, -inf once out of the running
   float* g_lds = rl + 2 * E;      // [groups] group scores
+  const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
   for (int e = lane; e < E; e += kWave) {
-    const float s = sigmoidf_(z[e]);
+    const float s = sigmoidf_(logits[t * E + e]);
     s_lds[e] = s;
     c_lds[e] = s + (correction != nullptr ? correction[e] : 0.0f);
     if (dense != nullptr) dense[t * E + e] = 0.0f;
@@ -199,42 +201,6 @@ __device__ __forceinline__ void route_token(const float* z, const float* __restr
     weights[t * top + lane] = w;
     if (dense != nullptr) dense[t * E + mine_id] = w;
   }
-}
-
-__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
-                                                        int32_t* __restrict__ ids, float* __restrict__ weights,
-                                                        float* __restrict__ dense, int E, int top, int groups, int keep,
-                                                        int normalize) {
-  extern __shared__ float rl[];
-  const int64_t t = blockIdx.x;
-  route_token(logits + t * E, correction, ids, weights, dense, t, E, top, groups, keep, normalize, rl);
-}
-
-// Router and choice in one launch, for steps of few tokens: one wave per token forms the E logits W_r h in f32 (the
-// token's row of activations widened to f32 in LDS, every expert's row of W_r read once, lanes striding over the width)
-// and then chooses from them.
-template <typename T>
-__global__ __launch_bounds__(64) void moe_router_route_kernel(const T* __restrict__ h, int64_t ld_h,
-                                                               const float* __restrict__ router_w,
-                                                               const float* __restrict__ correction, int32_t* __restrict__ ids,
-                                                               float* __restrict__ weights, float* __restrict__ dense, int W,
-                                                               int E, int top, int groups, int keep, int normalize, int ngroups) {
-  extern __shared__ float rl[];
-  float* z_lds = rl + 2 * E + ngroups;   // [E] logits
-  float* h_lds = z_lds + E;              // [W] the token's row
-  const int64_t t = blockIdx.x;
-  const int lane = threadIdx.x;
-  for (int i = lane; i < W; i += kWave) h_lds[i] = ldf(h + t * ld_h + i);
-  __syncthreads();
-  for (int e = 0; e < E; ++e) {
-    const float* wr = router_w + static_cast<int64_t>(e) * W;
-    float acc = 0.0f;
-    for (int i = lane; i < W; i += kWave) acc += h_lds[i] * wr[i];
-    acc = wave_sum(acc);
-    if (lane == 0) z_lds[e] = acc;
-  }
-  __syncthreads();
-  route_token(z_lds, correction, ids, weights, dense, t, E, top, groups, keep, normalize, rl);
 }
 
 template <typename T>
@@ -339,33 +305,6 @@ int lv_moe_route(const void* logits, const void* correction, void* ids, void* we
       static_cast<const float*>(logits), static_cast<const float*>(correction), static_cast<int32_t*>(ids),
       static_cast<float*>(weights), static_cast<float*>(dense), E, top, groups, keep, normalize);
   return launched("lv_moe_route");
-}
-
-int lv_moe_router_route(const void* h, int64_t ld_h, const void* router_w, const void* correction, void* ids, void* weights,
-                        void* dense, int64_t T, int W, int E, int top, int groups, int keep, int normalize, int dtype,
-                        void* stream) {
-  if (T == 0) return 0;
-  if (!h || !router_w || !ids || !weights || T < 0 || W <= 0 || ld_h < W || E <= 0 || top <= 0 || top > E || top > kWave)
-    return fail(-1, "lv_moe_router_route: bad arguments (experts %d, top %d, width %d)", E, top, W);
-  if (groups > 1 && (E % groups != 0 || keep <= 0 || keep > groups))
-    return fail(-1, "lv_moe_router_route: %d groups (keep %d) of %d experts", groups, keep, E);
-  const int ngroups = groups > 1 ? groups : 1;
-  const size_t shm = sizeof(float) * (3 * static_cast<size_t>(E) + static_cast<size_t>(ngroups) + static_cast<size_t>(W));
-  if (shm > 64 * 1024) return fail(-2, "lv_moe_router_route: %d experts at width %d need %zu bytes of LDS", E, W, shm);
-  dim3 grid(static_cast<unsigned>(T)), block(kWave);
-  if (dtype == LV_MIX_BF16)
-    moe_router_route_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<const bf16_t*>(h), ld_h, static_cast<const float*>(router_w), static_cast<const float*>(correction),
-        static_cast<int32_t*>(ids), static_cast<float*>(weights), static_cast<float*>(dense), W, E, top, groups, keep, normalize,
-        ngroups);
-  else if (dtype == LV_MIX_F32)
-    moe_router_route_kernel<float><<<grid, block, shm, as_stream(stream)>>>(
-        static_cast<const float*>(h), ld_h, static_cast<const float*>(router_w), static_cast<const float*>(correction),
-        static_cast<int32_t*>(ids), static_cast<float*>(weights), static_cast<float*>(dense), W, E, top, groups, keep, normalize,
-        ngroups);
-  else
-    return fail(-1, "lv_moe_router_route: dtype %d", dtype);
-  return launched("lv_moe_router_route");
 }
 
 int lv_relu2_scale(const void* up, const void* dense, void* out, int64_t T, int E, int F, int dtype, void* stream) {

@@ -651,29 +651,6 @@ def moe_route(logits, correction, top, groups=1, keep=1, normalize=True):
     return ids, w, dense
 
 
-ROUTER_FUSED_MAX_TOKENS = 256     # steps of at most this many tokens form their router logits inside the routing kernel
-
-
-def moe_router_route(h, router_w, correction, top, groups=1, keep=1, normalize=True):
-    """moe_route on logits = h router_w^T computed in f32 (h act [T, W], router_w f32 [E, W]). Steps of few tokens
-    (decoded tokens, small portions, everything replayed from a graph) form the logits inside the routing kernel, one
-    wave per token: one launch instead of a cast, a GEMM and the choice. Larger steps take the f32 vendor GEMM."""
-    T, W = h.shape
-    E = router_w.size(0)
-    _f32(router_w, correction)
-    if h.is_cuda and T <= ROUTER_FUSED_MAX_TOKENS and (3 * E + max(groups, 1) + W) * 4 <= 64 * 1024 and top <= 64:
-        assert h.stride(1) == 1
-        dev = h.device
-        ids = torch.empty(T, top, dtype=torch.int32, device=dev)
-        w = torch.empty(T, top, dtype=torch.float32, device=dev)
-        dense = torch.empty(T, E, dtype=torch.float32, device=dev)
-        lib = _mixlib.load()
-        _mixlib.check(lib.lv_moe_router_route(_p(h), h.stride(0), _p(router_w), _p(correction), _p(ids), _p(w), _p(dense), T, W, E,
-                                              top, groups, keep, int(normalize), _DT[h.dtype], _stream(h)), "lv_moe_router_route")
-        return ids, w, dense
-    return moe_route(F.linear(h.float(), router_w), correction, top, groups, keep, normalize)
-
-
 def relu2_scale(up, dense, E, Fe):
     """up act [T, E*Fe] (all experts' up projections), dense f32 [T, E] -> relu(up)^2 * dense[t, e], act."""
     T = up.size(0)
