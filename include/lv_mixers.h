@@ -22,6 +22,7 @@
  *   lv_latent_q_finish       joins the absorbed queries with their rotated positional part
  *   lv_latent_out_gate       per-head outputs [H, T, Dv] -> [T, H*Dv] times sigmoid(gate), gate per head or per channel
  *   lv_moe_route             sigmoid router with a selection-only correction, group limit and top-k
+ *   lv_router_logits         f32 router logits of steps of few tokens, straight from the activations
  *   lv_relu2_scale           squared relu of the experts' up projections times the routing weight
  *   lv_moe_grouped_ff        the experts' feed-forward on rows sorted by expert (grouped GEMMs on the matrix cores)
  *   lv_moe_sort, lv_moe_combine   its first and last step alone, for callers that multiply the sorted rows themselves
@@ -177,6 +178,11 @@ int lv_latent_out_gate(const void* o, const void* gate, int64_t ld_gate, int gat
  * ids int32 [T, top], weights f32 [T, top], dense f32 [T, E] (weights at the chosen experts, 0 elsewhere; may be NULL). */
 int lv_moe_route(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
                  int top, int groups, int keep, int normalize, void* stream);
+
+/* Router logits of steps of few tokens: logits f32 [T, E] = router_w h in f32 (h act [T, W] with row stride ld_h, router_w
+ * f32 [E, W]), without a widened copy of h; one workgroup per (token, four experts). */
+int lv_router_logits(const void* h, int64_t ld_h, const void* router_w, void* logits, int64_t T, int W, int E, int dtype,
+                     void* stream);
 
 /* up act [T, E*F] (all experts' up projections side by side), dense f32 [T, E]:
  * out act [T, E*F] = relu(up)^2 * dense[t, e]. */

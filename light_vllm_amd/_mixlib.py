@@ -46,6 +46,7 @@ SIGNATURES = {
     "lv_latent_q_finish": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
     "lv_latent_out_gate": (c_int, [_P, _P, c_int64, c_int, _P, c_int64, c_int, c_int, c_int, _P]),
     "lv_moe_route": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_router_logits": (c_int, [_P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, _P]),
     "lv_relu2_scale": (c_int, [_P, _P, _P, c_int64, c_int, c_int, c_int, _P]),
     "lv_moe_grouped_ff": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
     "lv_moe_grouped_workspace_bytes": (c_int64, [c_int64, c_int, c_int, c_int, c_int]),

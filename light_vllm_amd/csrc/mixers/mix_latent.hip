@@ -12,6 +12,8 @@
 //   latent_out_gate_kernel  elementwise: head-major outputs to token-major rows times sigmoid(gate).
 //   moe_route_kernel        one wave per token: sigmoid scores, correction for the choice only, group limit, top-k,
 //                           normalised (or raw) weights; the wave keeps its scores in LDS and picks maxima by shuffles.
+//   router_logits_kernel    steps of few tokens: the f32 router logits straight from the activations, one workgroup per
+//                           (token, four experts).
 //   relu2_scale_kernel      elementwise: relu(x)^2 times the token's weight for the expert the column belongs to.
 #include "mix_common.h"
 
@@ -203,6 +205,51 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
   }
 }
 
+// Router logits of steps of few tokens: one workgroup per (token, group of kRouterGroup experts) forms the dot products of
+// the token's row of activations with the experts' rows of the f32 router weight, in f32, without a widened copy of the
+// activations; four elements per access when the rows allow it.
+constexpr int kRouterGroup = 4;
+
+template <typename T, bool VEC4>
+__global__ __launch_bounds__(256) void router_logits_kernel(const T* __restrict__ h, int64_t ld_h, const float* __restrict__ router_w,
+                                                            float* __restrict__ logits, int W, int E) {
+  __shared__ float red[4][kRouterGroup];
+  const int64_t t = blockIdx.x;
+  const int e0 = blockIdx.y * kRouterGroup;
+  const T* row = h + t * ld_h;
+  float acc[kRouterGroup];
+#pragma unroll
+  for (int g = 0; g < kRouterGroup; ++g) acc[g] = 0.0f;
+  if constexpr (VEC4) {
+    for (int i = threadIdx.x * 4; i < W; i += blockDim.x * 4) {
+      const float4 x = ld4(row + i);
+#pragma unroll
+      for (int g = 0; g < kRouterGroup; ++g) {
+        if (e0 + g < E) {
+          const float4 w = ld4(router_w + static_cast<int64_t>(e0 + g) * W + i);
+          acc[g] += (x.x * w.x + x.y * w.y) + (x.z * w.z + x.w * w.w);
+        }
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      const float x = ldf(row + i);
+#pragma unroll
+      for (int g = 0; g < kRouterGroup; ++g)
+        if (e0 + g < E) acc[g] += x * router_w[static_cast<int64_t>(e0 + g) * W + i];
+    }
+  }
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+#pragma unroll
+  for (int g = 0; g < kRouterGroup; ++g) {
+    const float v = wave_sum(acc[g]);
+    if (lane == 0) red[wave][g] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < kRouterGroup && e0 + threadIdx.x < E)
+    logits[t * E + e0 + threadIdx.x] = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void relu2_scale_kernel(const T* __restrict__ up, const float* __restrict__ dense,
                                                           T* __restrict__ out, int64_t Tn, int E, int F) {
@@ -305,6 +352,28 @@ int lv_moe_route(const void* logits, const void* correction, void* ids, void* we
       static_cast<const float*>(logits), static_cast<const float*>(correction), static_cast<int32_t*>(ids),
       static_cast<float*>(weights), static_cast<float*>(dense), E, top, groups, keep, normalize);
   return launched("lv_moe_route");
+}
+
+int lv_router_logits(const void* h, int64_t ld_h, const void* router_w, void* logits, int64_t T, int W, int E, int dtype,
+                     void* stream) {
+  if (T == 0) return 0;
+  if (!h || !router_w || !logits || T < 0 || W <= 0 || E <= 0 || ld_h < W) return fail(-1, "lv_router_logits: bad arguments");
+  dim3 grid(static_cast<unsigned>(T), (E + kRouterGroup - 1) / kRouterGroup), block(256);
+  const bool vec4 = W % 4 == 0 && ld_h % 4 == 0 && (reinterpret_cast<uintptr_t>(h) & 15) == 0 &&
+                    (reinterpret_cast<uintptr_t>(router_w) & 15) == 0;
+#define LVMIX_ROUTER(TT, VV)                                                                                       \
+  router_logits_kernel<TT, VV><<<grid, block, 0, as_stream(stream)>>>(static_cast<const TT*>(h), ld_h,             \
+                                                                      static_cast<const float*>(router_w),         \
+                                                                      static_cast<float*>(logits), W, E)
+  if (dtype == LV_MIX_BF16) {
+    if (vec4) LVMIX_ROUTER(bf16_t, true); else LVMIX_ROUTER(bf16_t, false);
+  } else if (dtype == LV_MIX_F32) {
+    if (vec4) LVMIX_ROUTER(float, true); else LVMIX_ROUTER(float, false);
+  } else {
+    return fail(-1, "lv_router_logits: dtype %d", dtype);
+  }
+#undef LVMIX_ROUTER
+  return launched("lv_router_logits");
 }
 
 int lv_relu2_scale(const void* up, const void* dense, void* out, int64_t T, int E, int F, int dtype, void* stream) {

@@ -109,8 +109,7 @@ class GLUSparseMoE(nn.Module):
         self.down_weight = nn.Parameter(torch.empty(width, experts * ff + shared_ff))
 
     def route(self, h: torch.Tensor):
-        logits = F.linear(h.float(), self.router_weight)
-        return mix_ops.moe_route(logits, None, self.top, 1, 1, normalize=False)
+        return mix_ops.moe_route(mix_ops.router_logits(h, self.router_weight), None, self.top, 1, 1, normalize=False)
 
     def form(self, h: torch.Tensor) -> str:
         if MOE_KERNEL != "auto":

@@ -651,6 +651,26 @@ def moe_route(logits, correction, top, groups=1, keep=1, normalize=True):
     return ids, w, dense
 
 
+ROUTER_KERNEL_MAX_TOKENS = 256     # steps of at most this many tokens form their router logits in a kernel of their own
+
+
+def router_logits(h, router_w):
+    """f32 [T, E] = h router_w^T computed in f32 (h act [T, W], router_w f32 [E, W]). Steps of few tokens (decoded tokens,
+    small portions, everything replayed from a graph) read the activations as they are, one workgroup per (token, four
+    experts): one small launch instead of a widening copy and a GEMM. Larger steps take the f32 vendor GEMM."""
+    T, W = h.shape
+    E = router_w.size(0)
+    _f32(router_w)
+    if h.is_cuda and T <= ROUTER_KERNEL_MAX_TOKENS:
+        assert h.stride(1) == 1
+        logits = torch.empty(T, E, dtype=torch.float32, device=h.device)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_router_logits(_p(h), h.stride(0), _p(router_w), _p(logits), T, W, E, _DT[h.dtype], _stream(h)),
+                      "lv_router_logits")
+        return logits
+    return F.linear(h.float(), router_w)
+
+
 def relu2_scale(up, dense, E, Fe):
     """up act [T, E*Fe] (all experts' up projections), dense f32 [T, E] -> relu(up)^2 * dense[t, e], act."""
     T = up.size(0)

@@ -210,6 +210,21 @@ def case_moe_route_raw(device):
         assert torch.equal(ids.cpu().long(), want.indices[:, :top]) and torch.allclose(w.cpu(), want.values[:, :top], rtol=1e-6)
 
 
+def case_router_logits(device):
+    """The router's f32 logits from bf16 and f32 activations, in the kernel of small steps and through the GEMM of large
+    ones, rows of a wider tensor, widths that are no multiple of four, expert counts that are no multiple of the group."""
+    from light_vllm_amd import mix_ops
+    g = torch.Generator().manual_seed(6)
+    for T, W, E, dt in ((7, 48, 6, torch.float32), (40, 200, 33, torch.bfloat16), (300, 64, 8, torch.bfloat16),
+                        (3, 1001, 5, torch.float32), (16, 2048, 32, torch.bfloat16), (5, 30, 1, torch.bfloat16)):
+        buf = torch.randn(T, W + 8, generator=g).to(dt)
+        rw = torch.randn(E, W, generator=g) / W ** 0.5
+        want = buf[:, 8:].to(F64) @ rw.to(F64).T
+        for hd in (buf.to(device)[:, 8:], buf[:, 8:].contiguous().to(device)):
+            got = mix_ops.router_logits(hd, rw.to(device)).cpu().to(F64)
+            assert got.shape == (T, E) and (got - want).abs().max().item() <= 2e-5 * max(1.0, want.abs().max().item()), (T, W, E, dt)
+
+
 def case_moe_ff(device, dtype):
     """The mixture with gated experts in both forms against the oracle: the weight scales the expert's INPUT (with a small
     clamp the two readings differ by far), the shared expert and its token gate, every expert chosen, one expert."""

@@ -24,6 +24,10 @@ def test_moe_route_raw():
     C.case_moe_route_raw(DEV)
 
 
+def test_router_logits():
+    C.case_router_logits(DEV)
+
+
 def test_attention_beacons():
     C.case_attention_beacons(DEV, "float32")
 

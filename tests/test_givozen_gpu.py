@@ -25,6 +25,10 @@ def test_moe_route_raw(gpu):
     C.case_moe_route_raw(DEV)
 
 
+def test_router_logits(gpu):
+    C.case_router_logits(DEV)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_beacons(gpu, dtype):
     C.case_attention_beacons(DEV, dtype)

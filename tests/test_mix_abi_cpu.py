@@ -57,6 +57,7 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.lv_polynorm(p, 8, p, p, 1, 8, 1e-6, 7, None) == -1                      # unknown dtype
     assert lib.lv_expert_glu(p, 8, None, None, 0, p, 8, 1, 2, 8, 1.0, 1.702, 0, None) == -1     # two experts need 32 columns
     assert lib.lv_moe_route(p, None, p, p, None, 1, 4, 5, 1, 1, 0, None) == -1                 # more choices than experts
+    assert lib.lv_router_logits(p, 4, p, p, 1, 8, 4, 0, None) == -1                            # row stride below the row
     assert lib.lv_moe_grouped_glu_ff(p, p, p, p, p, 0, p, p, 1, 48, 32, 4, 2, 1.0, 1.702, None) == -1     # width no multiple of 32
     assert lib.lv_moe_grouped_glu_ff(p, p, p, p, p, 100, p, p, 1, 64, 32, 4, 2, 1.0, 1.702, None) == -1   # down rows shorter than E*F
     assert lib.lv_window_pool_attn(p, p, p, None, None, p, 4, p, p, p, p, p, 1, 1, 4, 2, 8, 8, 16, 64, 0, 0.5, 0, 0, 0, 5, 0, None) == -1   # gate kind
