@@ -48,6 +48,7 @@ class GivozenConfig:
     loop_start: int = 0
     loop_stop: int = 0
     loop_times: int = 1
+    has_loop: bool = False                       # the config names a loop (its table of pass vectors exists even if the stretch is empty)
     torch_dtype: Any = torch.bfloat16
     max_position_embeddings: int = 1 << 30       # positions are rotated on the fly: any length the cache holds
     architectures: tuple = ("Givozen",)
@@ -110,7 +111,7 @@ class GivozenConfig:
         if loop and not (0 <= start <= stop <= len(layers) and times >= 1):
             raise ValueError(f"loop {loop} does not fit {len(layers)} layers")
         return cls(vocab=int(d["vocab"]), width=int(d["width"]), norm_eps=float(d["norm"]["eps"]), layers=layers,
-                   loop_start=start, loop_stop=stop, loop_times=times)
+                   loop_start=start, loop_stop=stop, loop_times=times, has_loop=bool(loop))
 
     @classmethod
     def from_pretrained(cls, path: str) -> "GivozenConfig":
@@ -193,7 +194,7 @@ class GivozenForCausalLM(nn.Module):
                 self.repeats.append(layer)
             seen.add(i)
             self.order.append((layer, t))
-        self.loop_step = nn.Parameter(torch.zeros(config.loop_times, config.width, dtype=torch.float32)) if config.looped else None
+        self.loop_step = nn.Parameter(torch.zeros(config.loop_times, config.width, dtype=torch.float32)) if config.has_loop else None
         self.final_norm = OffsetNormWeight(config.width)
         self.lm_head = ParallelLMHead(config.vocab, config.width)
         self.lm_head.weight = self.embed.weight    # the output head is the embedding table
@@ -346,6 +347,8 @@ class GivozenForCausalLM(nn.Module):
                 param.copy_(torch.tensor([0.6, 0.3, 0.1, 0.0]))
             else:
                 param.normal_(0.0, std, generator=g)
+        for layer in self.layers:           # the gate's part of the merged bias has no tensor: it is zero
+            layer.mix.in_proj.bias[sum(layer.mix.sizes[:3]):].zero_()
 
     def random_weights(self, seed: int = 0):
         """(name, tensor) pairs of a seeded random checkpoint of this configuration, for runs without
