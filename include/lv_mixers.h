@@ -35,6 +35,17 @@
  *                            on the pre-activations and a sigmoid per token on the result
  *   lv_moe_grouped_glu_ff    the gathered feed-forward for clamped gated experts whose routing weight scales the
  *                            expert's input
+ *   lv_residual_dyt          single f32 residual: adds a sublayer output, or the scaled sum of two RMS-normed and weighted
+ *                            ones (two mixers side by side), then the dynamic-tanh norm tanh(alpha x) w + b
+ *   lv_qk_prep_store         lv_rotary_store with the pairing of rotated entries as a choice and an optional division of
+ *                            every query and key head by its root mean square
+ *   lv_masked_attn(_mfma)    lv_window_pool_attn(_mfma) with kept first tokens, chunked visibility and a learned sink per head
+ *   lv_lightning_attn        linear attention with a constant decay per head: S <- d S + k v^T, o = S^T q, state in f32
+ *   lv_glu_act               act(gate) * up
+ *   lv_moe_route_scored      lv_moe_route with softmax scores and groups ranked by their best expert as choices
+ *   lv_expert_act_scale      lv_relu2_scale with the activation as a choice
+ *   lv_moe_grouped_act_ff    lv_moe_grouped_ff with the activation as a choice and experts that hand their input through
+ *   lv_scaled_row_add        y[t] += (sum of a token's factors) * h[t]
  *
  * A "ragged step" is a batch of B sequences; sequence b brings cu_q[b+1]-cu_q[b] new tokens that
  * follow ctx_lens[b] tokens already in the cache / state (a whole prompt, a portion of one, or one
@@ -56,7 +67,7 @@
 extern "C" {
 #endif
 
-#define LV_MIX_ABI_VERSION 6
+#define LV_MIX_ABI_VERSION 7
 #define LV_MIX_BF16 0
 #define LV_MIX_F32 1
 #define LV_MIX_MAX_STREAMS 8
@@ -64,6 +75,13 @@ extern "C" {
 #define LV_MIX_GATE_SIGMOID 1
 #define LV_MIX_GATE_PER_HEAD 0
 #define LV_MIX_GATE_PER_CHANNEL 1
+#define LV_MIX_ACT_RELU2 0        /* relu(z)^2 */
+#define LV_MIX_ACT_GELU_ERF 1     /* z Phi(z), exact */
+#define LV_MIX_ACT_GELU_TANH 2    /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */
+#define LV_MIX_SCORE_SIGMOID 0
+#define LV_MIX_SCORE_SOFTMAX 1
+#define LV_MIX_GROUP_TOP2_SUM 0   /* a group of experts is ranked by the sum of its two highest selection scores */
+#define LV_MIX_GROUP_MAX 1        /* ... by its highest */
 
 int lv_mix_abi_version(void);
 const char* lv_mix_last_error(void);
@@ -243,6 +261,70 @@ int lv_expert_glu(const void* in, int64_t ld_in, const void* in_scale, const voi
 int lv_moe_grouped_glu_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w,
                           int64_t down_ld, void* out, void* workspace, int64_t T, int W, int F, int E, int top, float limit,
                           float alpha, void* stream);
+
+/* x f32 [T, W] in place.  post_w1 == NULL:  x += y1 + y2                  (act [T, W]; either may be NULL)
+ *                         post_w1 != NULL:  x += pair_scale * (y1 / rms(y1) * post_w1 + y2 / rms(y2) * post_w2)
+ *                                           (rms(y) = sqrt(mean(y^2) + eps); y2 with post_w2 may be NULL)
+ * out act [T, W] = tanh(alpha[0] * x) * w + b  (alpha f32 [1], w and b f32 [W]; out may be NULL: update only). All f32. */
+int lv_residual_dyt(void* x, const void* y1, const void* post_w1, const void* y2, const void* post_w2, float pair_scale,
+                    float eps, const void* alpha, const void* w, const void* b, void* out, int64_t T, int W, int dtype,
+                    void* stream);
+
+/* lv_rotary_store with two more choices. interleaved != 0: rotated entry 2i pairs with 2i + 1 (else i with i + rot_dims/2),
+ * angle = position * inv_freq[i]. unit_norm != 0: every query and key head is divided by sqrt(mean(head^2) + eps) (no weight). */
+int lv_qk_prep_store(const void* proj, int64_t ld, int off_q, int off_k, int off_v, const void* inv_freq,
+                     const void* head_scale, void* q_out, void* k_cache, void* v_cache, const int32_t* cu_q,
+                     const int32_t* ctx_lens, const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T,
+                     int H, int G, int D, int Dv, int rot_dims, int interleaved, int unit_norm, float eps, int page, int dtype,
+                     void* stream);
+
+/* lv_window_pool_attn with more ways to say what a query at position i sees among the cached positions j <= i:
+ *   chunk == 0: i - j < window or j < keep_first;   chunk > 0: floor(i / chunk) == floor(j / chunk) or j < keep_first
+ * (kept first tokens and chunks do not combine with pooled blocks, P > 0). sinks f32 [H] (may be NULL): the denominator of
+ * head h's softmax also holds exp(sinks[h]); has_sink without sinks: exp(0). */
+int lv_masked_attn(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
+                   const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
+                   const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G, int D,
+                   int Dv, int page, int window, int keep_first, int chunk, int P, float scale, int has_sink,
+                   const void* sinks, int64_t k_ld, int64_t v_ld, int gate_kind, int dtype, void* stream);
+int lv_masked_attn_mfma(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
+                        const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
+                        const int32_t* block_tables, int bt_stride, int B, int max_new_tokens, int H, int G, int D,
+                        int Dv, int page, int window, int keep_first, int chunk, int P, float scale, int has_sink,
+                        const void* sinks, int nsplit, void* workspace, int64_t T, int64_t k_ld, int64_t v_ld,
+                        int gate_kind, void* stream);
+
+/* proj act [T, ld]: H query heads of D at column off_q, H key heads of D at off_k, H value heads of Dv at off_v; each entry
+ * passes silu first. Per head and token: S <- decay[h] * S + k v^T; o = S^T q. state f32 [slots, H, D, Dv], read unless
+ * ctx_lens[b] == 0, written back; decay f32 [H]; o f32 [T, H, Dv]. */
+int lv_lightning_attn(const void* proj, int64_t ld, int off_q, int off_k, int off_v, const void* decay, void* state,
+                      const int32_t* cu_q, const int32_t* ctx_lens, const int32_t* slots, void* o, int B, int H, int D, int Dv,
+                      int dtype, void* stream);
+
+/* in act [T, 2F] (row stride ld_in) = [gate | up];  out act [T, F] = act(gate) * up, act one of LV_MIX_ACT_*. */
+int lv_glu_act(const void* in, int64_t ld_in, void* out, int64_t T, int F, int act, int dtype, void* stream);
+
+/* lv_moe_route with the scores as sigmoid or as softmax over all E logits of the row (LV_MIX_SCORE_*), and the rank of a
+ * group as the sum of its two highest selection scores or its highest (LV_MIX_GROUP_*). */
+int lv_moe_route_scored(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
+                        int top, int groups, int keep, int normalize, int score_kind, int group_rank, void* stream);
+
+/* up act [T, E*F], dense f32 rows of stride ld_dense (>= E):  out act [T, E*F] = act(up) * dense[t, e], 0 where dense is 0. */
+int lv_expert_act_scale(const void* up, const void* dense, int64_t ld_dense, void* out, int64_t T, int E, int F, int act,
+                        int dtype, void* stream);
+
+/* lv_moe_grouped_ff with the activation as a choice and n_through more expert numbers (E_real .. E_real + n_through - 1)
+ * that stand for no weights: such a choice contributes weight * h[t]. ids hold numbers below E_real + n_through;
+ * workspace: lv_moe_grouped_workspace_bytes(T, W, F, E_real + n_through, top). */
+int lv_moe_grouped_act_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w, void* out,
+                          void* workspace, int64_t T, int W, int F, int E_real, int n_through, int top, int act, void* stream);
+/* lv_moe_combine in which a choice with ids[t, k] >= n_real takes the row h[t] (bf16 [T, W]) instead of a row of `rows`. */
+int lv_moe_combine_through(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top,
+                           const void* ids, int n_real, const void* h, void* stream);
+
+/* y act [T, W] += (factors[t, 0] + ... + factors[t, nf - 1]) * h[t]; factors f32 rows of stride ld_f. */
+int lv_scaled_row_add(void* y, const void* h, const void* factors, int64_t ld_f, int nf, int64_t T, int W, int dtype,
+                      void* stream);
 
 #ifdef __cplusplus
 }

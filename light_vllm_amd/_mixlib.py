@@ -17,8 +17,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc", "mixers")
 LIB_PATH = os.path.join(_HERE, "lib", "liblvmix.so")
 SOURCES = ["mix_stream.hip", "mix_window_attn.hip", "mix_window_mfma.hip", "mix_latent.hip", "mix_moe_gemm.hip",
-           "mix_sandwich.hip"]
-ABI_VERSION = 6
+           "mix_sandwich.hip", "mix_parallel.hip"]
+ABI_VERSION = 7
 
 _P = c_void_p
 SIGNATURES = {
@@ -59,6 +59,21 @@ SIGNATURES = {
     "lv_expert_glu": (c_int, [_P, c_int64, _P, _P, c_int64, _P, c_int64, c_int64, c_int, c_int, c_float, c_float, c_int, _P]),
     "lv_moe_grouped_glu_ff": (c_int, [_P, _P, _P, _P, _P, c_int64, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_float,
                                       c_float, _P]),
+    "lv_residual_dyt": (c_int, [_P, _P, _P, _P, _P, c_float, c_float, _P, _P, _P, _P, c_int64, c_int, c_int, _P]),
+    "lv_qk_prep_store": (c_int, [_P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int64,
+                                 c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P]),
+    "lv_masked_attn": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, _P, c_int, c_int64, c_int, c_int, c_int, c_int,
+                               c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P, c_int64, c_int64, c_int, c_int, _P]),
+    "lv_masked_attn_mfma": (c_int, [_P, _P, _P, _P, _P, _P, c_int64, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P, c_int, _P, c_int64, c_int64,
+                                    c_int64, c_int, _P]),
+    "lv_lightning_attn": (c_int, [_P, c_int64, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_glu_act": (c_int, [_P, c_int64, _P, c_int64, c_int, c_int, c_int, _P]),
+    "lv_moe_route_scored": (c_int, [_P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_expert_act_scale": (c_int, [_P, _P, c_int64, _P, c_int64, c_int, c_int, c_int, c_int, _P]),
+    "lv_moe_grouped_act_ff": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lv_moe_combine_through": (c_int, [_P, _P, _P, _P, c_int64, c_int, c_int, _P, c_int, _P, _P]),
+    "lv_scaled_row_add": (c_int, [_P, _P, _P, c_int64, c_int, c_int64, c_int, c_int, _P]),
 }
 
 _lib = None

@@ -136,15 +136,23 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ correction,
                                                         int32_t* __restrict__ ids, float* __restrict__ weights,
                                                         float* __restrict__ dense, int E, int top, int groups, int keep,
-                                                        int normalize) {
+                                                        int normalize, int score_kind, int group_rank) {
   extern __shared__ float rl[];
   float* s_lds = rl;              // [E] scores
   float* c_lds = rl + E;          // [E] selection scores, -inf once out of the running
   float* g_lds = rl + 2 * E;      // [groups] group scores
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
+  float smax = -INFINITY, sden = 1.0f;
+  if (score_kind == LV_MIX_SCORE_SOFTMAX) {            // over all experts of the row
+    for (int e = lane; e < E; e += kWave) smax = fmaxf(smax, logits[t * E + e]);
+    smax = wave_max(smax);
+    float part = 0.0f;
+    for (int e = lane; e < E; e += kWave) part += expf(logits[t * E + e] - smax);
+    sden = wave_sum(part);
+  }
   for (int e = lane; e < E; e += kWave) {
-    const float s = sigmoidf_(logits[t * E + e]);
+    const float s = score_kind == LV_MIX_SCORE_SOFTMAX ? expf(logits[t * E + e] - smax) / sden : sigmoidf_(logits[t * E + e]);
     s_lds[e] = s;
     c_lds[e] = s + (correction != nullptr ? correction[e] : 0.0f);
     if (dense != nullptr) dense[t * E + e] = 0.0f;
@@ -159,7 +167,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
         if (c > a) { b2 = a; a = c; }
         else if (c > b2) b2 = c;
       }
-      g_lds[g] = gs > 1 ? a + b2 : a;
+      g_lds[g] = (gs > 1 && group_rank == LV_MIX_GROUP_TOP2_SUM) ? a + b2 : a;
     }
     __syncthreads();
     // the `keep` best groups: their score is marked +inf, everything else leaves the choice
@@ -341,7 +349,16 @@ int lv_latent_out_gate(const void* o, const void* gate, int64_t ld_gate, int gat
 
 int lv_moe_route(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
                  int top, int groups, int keep, int normalize, void* stream) {
+  return lv_moe_route_scored(logits, correction, ids, weights, dense, T, E, top, groups, keep, normalize, LV_MIX_SCORE_SIGMOID,
+                             LV_MIX_GROUP_TOP2_SUM, stream);
+}
+
+int lv_moe_route_scored(const void* logits, const void* correction, void* ids, void* weights, void* dense, int64_t T, int E,
+                        int top, int groups, int keep, int normalize, int score_kind, int group_rank, void* stream) {
   if (T == 0) return 0;
+  if ((score_kind != LV_MIX_SCORE_SIGMOID && score_kind != LV_MIX_SCORE_SOFTMAX) ||
+      (group_rank != LV_MIX_GROUP_TOP2_SUM && group_rank != LV_MIX_GROUP_MAX))
+    return fail(-1, "lv_moe_route: score kind %d, group rank %d", score_kind, group_rank);
   if (!logits || !ids || !weights || T < 0 || E <= 0 || top <= 0 || top > E || top > kWave)
     return fail(-1, "lv_moe_route: bad arguments (experts %d, top %d)", E, top);
   if (groups > 1 && (E % groups != 0 || keep <= 0 || keep > groups))
@@ -350,7 +367,7 @@ int lv_moe_route(const void* logits, const void* correction, void* ids, void* we
   if (shm > 64 * 1024) return fail(-2, "lv_moe_route: %d experts need %zu bytes of LDS", E, shm);
   moe_route_kernel<<<dim3(static_cast<unsigned>(T)), dim3(kWave), shm, as_stream(stream)>>>(
       static_cast<const float*>(logits), static_cast<const float*>(correction), static_cast<int32_t*>(ids),
-      static_cast<float*>(weights), static_cast<float*>(dense), E, top, groups, keep, normalize);
+      static_cast<float*>(weights), static_cast<float*>(dense), E, top, groups, keep, normalize, score_kind, group_rank);
   return launched("lv_moe_route");
 }
 

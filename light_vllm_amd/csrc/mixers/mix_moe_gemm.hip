@@ -82,6 +82,8 @@ struct MoeGemmParams {
   int64_t b_expert;        // elements from one expert's B to the next
   const float* row_scale;  // GLU: [pairs] factor on the pre-activations of a (token, choice) pair
   float limit, alpha;      // GLU: clamp and sigmoid slope of the gated unit
+  int act;                 // UP without GLU: LV_MIX_ACT_* applied to the product
+  int n_real;              // tiles of buckets from this number on have no weights (experts that hand their input through) and are skipped
 };
 
 // MB x NB blocks of 16 x 16 per wave; WM waves along the rows (1 or 2), the others along the columns: the workgroup's
@@ -103,6 +105,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
   const int ln = lane & 15, lg = lane >> 4;
   const int wm = wave % WM, wn = wave / WM;
   const int e = p.tiles[3 * tile], row0 = p.tiles[3 * tile + 1], nrows = p.tiles[3 * tile + 2];
+  if (e >= p.n_real) return;
   const int m0 = wm * 16 * MB;
   const int n0 = (bx * (4 / WM) + wn) * 16 * CB;
   if (n0 >= p.N || m0 >= nrows) return;
@@ -181,8 +184,14 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
         } else {
           v = acc[mb][nb][i];
           if (UP) {
-            v = fmaxf(v, 0.0f);
-            v = v * v;
+            if (p.act == LV_MIX_ACT_GELU_ERF) {
+              v = 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
+            } else if (p.act == LV_MIX_ACT_GELU_TANH) {
+              v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+            } else {
+              v = fmaxf(v, 0.0f);
+              v = v * v;
+            }
           }
         }
         bf16_t t;
@@ -195,15 +204,19 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(MoeGemmParams p) {
   }
 }
 
+// ids, n_real, h (all or none): a choice whose expert number is n_real or above hands the token's own row h[t] through
+// instead of a row of `rows`.
 __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t* __restrict__ rows, const int32_t* __restrict__ inv,
                                                           const float* __restrict__ weights, uint16_t* __restrict__ out,
-                                                          int W, int top) {
+                                                          int W, int top, const int32_t* __restrict__ ids, int n_real,
+                                                          const uint16_t* __restrict__ h) {
   const int64_t t = blockIdx.x;
   for (int c = threadIdx.x * 4; c < W; c += blockDim.x * 4) {
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int k = 0; k < top; ++k) {
       const float w = weights != nullptr ? weights[t * top + k] : 1.0f;
-      const uint2 v = *reinterpret_cast<const uint2*>(rows + static_cast<int64_t>(inv[t * top + k]) * W + c);
+      const bool through = ids != nullptr && ids[t * top + k] >= n_real;
+      const uint2 v = *reinterpret_cast<const uint2*>(through ? h + t * W + c : rows + static_cast<int64_t>(inv[t * top + k]) * W + c);
       acc[0] += w * __builtin_bit_cast(float, v.x << 16);
       acc[1] += w * __builtin_bit_cast(float, v.x & 0xffff0000u);
       acc[2] += w * __builtin_bit_cast(float, v.y << 16);
@@ -255,9 +268,16 @@ int lv_moe_max_tiles(int64_t pairs, int E, int BM) {
 
 int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w, void* out,
                       void* workspace, int64_t T, int W, int F, int E, int top, void* stream) {
+  return lv_moe_grouped_act_ff(h, ids, weights, up_w, down_w, out, workspace, T, W, F, E, 0, top, LV_MIX_ACT_RELU2, stream);
+}
+
+int lv_moe_grouped_act_ff(const void* h, const void* ids, const void* weights, const void* up_w, const void* down_w, void* out,
+                          void* workspace, int64_t T, int W, int F, int E_real, int n_through, int top, int act, void* stream) {
   if (T == 0) return 0;
   if (!h || !ids || !weights || !up_w || !down_w || !out || !workspace) return fail(-1, "lv_moe_grouped_ff: null pointer");
-  if (T < 0 || W <= 0 || F <= 0 || E <= 0 || top <= 0 || W % 32 != 0 || F % 32 != 0 || E > 4096)
+  const int E = E_real + n_through;                 // buckets of the sort; the last n_through have no weights
+  if (T < 0 || W <= 0 || F <= 0 || E_real <= 0 || n_through < 0 || top <= 0 || W % 32 != 0 || F % 32 != 0 || E > 4096 ||
+      act < 0 || act > LV_MIX_ACT_GELU_TANH)
     return fail(-1, "lv_moe_grouped_ff: width %d and expert size %d must be multiples of 32 (experts %d)", W, F, E);
   const int64_t M = T * top;
   if (M > (1 << 30)) return fail(-2, "lv_moe_grouped_ff: %lld rows", (long long)M);
@@ -269,20 +289,21 @@ int lv_moe_grouped_ff(const void* h, const void* ids, const void* weights, const
   int32_t* tiles = inv + M;
   int32_t* num_tiles = tiles + 3 * static_cast<int64_t>(max_tiles);
   const int64_t ints = (2 * M + 3 * static_cast<int64_t>(max_tiles) + 1 + 3) / 4 * 4;
-  uint16_t* act = reinterpret_cast<uint16_t*>(sorted_pair + ints);
-  uint16_t* rows = act + M * F;
+  uint16_t* act_rows = reinterpret_cast<uint16_t*>(sorted_pair + ints);
+  uint16_t* rows = act_rows + M * F;
   hipStream_t s = as_stream(stream);
   const size_t shm = sizeof(int32_t) * (3 * static_cast<size_t>(E) + 2);
   moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, s>>>(static_cast<const int32_t*>(ids), static_cast<int>(M), E, BM,
                                                           sorted_pair, inv, tiles, num_tiles, max_tiles, nullptr, 1);
-  MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act, sorted_pair, tiles, num_tiles,
-                   F, W, top, W, W, F, static_cast<int64_t>(F) * W, nullptr, 0.0f, 0.0f};
+  MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act_rows, sorted_pair, tiles, num_tiles,
+                   F, W, top, W, W, F, static_cast<int64_t>(F) * W, nullptr, 0.0f, 0.0f, act, E_real};
   gemm_launch<true>(up, max_tiles, BM, s);
-  MoeGemmParams down{act, static_cast<const uint16_t*>(down_w), rows, sorted_pair, tiles, num_tiles,
-                     W, F, top, F, static_cast<int64_t>(E) * F, W, F, nullptr, 0.0f, 0.0f};
+  MoeGemmParams down{act_rows, static_cast<const uint16_t*>(down_w), rows, sorted_pair, tiles, num_tiles,
+                     W, F, top, F, static_cast<int64_t>(E_real) * F, W, F, nullptr, 0.0f, 0.0f, 0, E_real};
   gemm_launch<false>(down, max_tiles, BM, s);
-  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, static_cast<const float*>(weights),
-                                                                          static_cast<uint16_t*>(out), W, top);
+  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(
+      rows, inv, static_cast<const float*>(weights), static_cast<uint16_t*>(out), W, top,
+      n_through > 0 ? static_cast<const int32_t*>(ids) : nullptr, E_real, static_cast<const uint16_t*>(h));
   return launched("lv_moe_grouped_ff");
 }
 
@@ -314,12 +335,12 @@ int lv_moe_grouped_glu_ff(const void* h, const void* ids, const void* weights, c
   moe_sort_kernel<<<dim3(1), dim3(kSortThreads), shm, s>>>(static_cast<const int32_t*>(ids), static_cast<int>(M), E, BM,
                                                           sorted_pair, inv, tiles, num_tiles, max_tiles, nullptr, 1);
   MoeGemmParams up{static_cast<const uint16_t*>(h), static_cast<const uint16_t*>(up_w), act, sorted_pair, tiles, num_tiles,
-                   F, W, top, W, W, F, 2 * static_cast<int64_t>(F) * W, static_cast<const float*>(weights), limit, alpha};
+                   F, W, top, W, W, F, 2 * static_cast<int64_t>(F) * W, static_cast<const float*>(weights), limit, alpha, 0, E};
   gemm_launch<true, true>(up, max_tiles, BM, s);
   MoeGemmParams down{act, static_cast<const uint16_t*>(down_w), rows, sorted_pair, tiles, num_tiles,
-                     W, F, top, F, down_ld, W, F, nullptr, 0.0f, 0.0f};
+                     W, F, top, F, down_ld, W, F, nullptr, 0.0f, 0.0f, 0, E};
   gemm_launch<false>(down, max_tiles, BM, s);
-  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, nullptr, static_cast<uint16_t*>(out), W, top);
+  moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, s>>>(rows, inv, nullptr, static_cast<uint16_t*>(out), W, top, nullptr, 0, nullptr);
   return launched("lv_moe_grouped_glu_ff");
 }
 
@@ -335,11 +356,17 @@ int lv_moe_sort(const void* ids, int64_t M, int E, int align, void* sorted_pair,
 }
 
 int lv_moe_combine(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top, void* stream) {
+  return lv_moe_combine_through(rows, inv, weights, out, T, W, top, nullptr, 0, nullptr, stream);
+}
+
+int lv_moe_combine_through(const void* rows, const void* inv, const void* weights, void* out, int64_t T, int W, int top,
+                           const void* ids, int n_real, const void* h, void* stream) {
   if (T == 0) return 0;
-  if (!rows || !inv || !out || T < 0 || W <= 0 || W % 4 != 0 || top <= 0) return fail(-1, "lv_moe_combine: bad arguments");
+  if (!rows || !inv || !out || T < 0 || W <= 0 || W % 4 != 0 || top <= 0 || ((ids != nullptr) != (h != nullptr)))
+    return fail(-1, "lv_moe_combine: bad arguments");
   moe_combine_kernel<<<dim3(static_cast<unsigned>(T)), dim3(256), 0, as_stream(stream)>>>(
       static_cast<const uint16_t*>(rows), static_cast<const int32_t*>(inv), static_cast<const float*>(weights),
-      static_cast<uint16_t*>(out), W, top);
+      static_cast<uint16_t*>(out), W, top, static_cast<const int32_t*>(ids), n_real, static_cast<const uint16_t*>(h));
   return launched("lv_moe_combine");
 }
 

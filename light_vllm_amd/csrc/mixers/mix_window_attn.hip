@@ -86,6 +86,9 @@ struct WindowAttnParams {
   float scale, sink;
   int64_t k_ld, v_ld;   // elements between the rows of two cached tokens (G*D and G*Dv unless the caches are views of wider rows)
   float m0;             // where the running maximum starts: the sink's score 0, or far below any score without a sink
+  int keep_first;       // positions below this are seen from everywhere (with their own keys and values)
+  int chunk;            // > 0: a query sees its own chunk of that many positions (counted from 0) up to itself; no window
+  const float* sinks;   // [H] or NULL: a learned score per query head in place of the sink's 0
 };
 
 // kMaxRep: query heads of one kv head served by one workgroup; kMaxDvi: value columns per lane (Dv <= 64 * kMaxDvi).
@@ -112,10 +115,11 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
   const int b = p.tok_seq[t];
   const int pos = p.ctx_lens[b] + static_cast<int>(t) - p.cu_q[b];
   const int32_t* bt = p.block_tables + static_cast<int64_t>(b) * p.bt_stride;
-  const int j0 = max(0, pos - p.window + 1);
+  const int j0 = p.chunk > 0 ? (pos / p.chunk) * p.chunk : max(0, pos - p.window + 1);
   const int nw = pos - j0 + 1;
-  const int nb = (p.P > 0 && pos - p.window + 1 > 0) ? (pos - p.window + 1) / p.P : 0;
-  const int nkeys = nb + nw;
+  const int nb = (p.P > 0 && p.chunk == 0 && pos - p.window + 1 > 0) ? (pos - p.window + 1) / p.P : 0;
+  const int nf = min(p.keep_first, j0);                 // kept first tokens that lie before the window
+  const int nkeys = nb + nf + nw;                       // [pooled blocks | kept first tokens | window]
   const int GD = p.G * D, GDv = p.G * Dv;
   const T* kc = static_cast<const T*>(p.k_cache);
   const T* vc = static_cast<const T*>(p.v_cache);
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
   float m[kMaxRep], l[kMaxRep], o[kMaxRep][kMaxDvi];
 #pragma unroll
   for (int h = 0; h < kMaxRep; ++h) {
-    m[h] = p.m0;                                        // with a sink: never below its score
+    m[h] = (p.sinks != nullptr && h < rep) ? p.sinks[h0 + h] : p.m0;   // with a sink: never below its score
     l[h] = wave == 0 ? p.sink : 0.0f;
 #pragma unroll
     for (int e = 0; e < kMaxDvi; ++e) o[h][e] = 0.0f;
@@ -142,7 +146,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
         const int pj = (idx * p.P + p.P - 1) / p.page;
         krow = kpool + (static_cast<int64_t>(bt[pj]) * p.PP + (idx - (p.page * pj) / p.P)) * GD + g * D;
       } else {
-        const int j = j0 + idx - nb;
+        const int j = idx < nb + nf ? idx - nb : j0 + idx - nb - nf;
         krow = kc + (static_cast<int64_t>(bt[j / p.page]) * p.page + j % p.page) * p.k_ld + g * D;
       }
     }
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
         const int pj = (id2 * p.P + p.P - 1) / p.page;
         vrow = vpool + (static_cast<int64_t>(bt[pj]) * p.PP + (id2 - (p.page * pj) / p.P)) * GDv + g * Dv;
       } else {
-        const int j = j0 + id2 - nb;
+        const int j = id2 < nb + nf ? id2 - nb : j0 + id2 - nb - nf;
         vrow = vc + (static_cast<int64_t>(bt[j / p.page]) * p.page + j % p.page) * p.v_ld + g * Dv;
       }
 #pragma unroll
@@ -215,7 +219,7 @@ __global__ __launch_bounds__(256) void window_pool_attn_kernel(WindowAttnParams 
   const T* gate = p.gate != nullptr ? static_cast<const T*>(p.gate) + t * p.ld_gate : nullptr;
   for (int i = threadIdx.x; i < rep * Dv; i += blockDim.x) {
     const int h = i / Dv, dv = i - h * Dv;
-    float mm = p.m0;
+    float mm = p.sinks != nullptr ? p.sinks[h0 + h] : p.m0;
     for (int w = 0; w < 4; ++w) mm = fmaxf(mm, ml_lds[(w * kMaxRep + h) * 2]);
     float ll = 0.0f, acc = 0.0f;
     for (int w = 0; w < 4; ++w) {
@@ -289,7 +293,19 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
                         const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G, int D,
                         int Dv, int page, int window, int P, float scale, int has_sink, int64_t k_ld, int64_t v_ld,
                         int gate_kind, int dtype, void* stream) {
+  return lv_masked_attn(q, k_cache, v_cache, kp, vp, gate, ld_gate, out, cu_q, ctx_lens, tok_seq, block_tables, bt_stride, T, H,
+                        G, D, Dv, page, window, 0, 0, P, scale, has_sink, nullptr, k_ld, v_ld, gate_kind, dtype, stream);
+}
+
+int lv_masked_attn(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
+                   const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
+                   const int32_t* tok_seq, const int32_t* block_tables, int bt_stride, int64_t T, int H, int G, int D,
+                   int Dv, int page, int window, int keep_first, int chunk, int P, float scale, int has_sink,
+                   const void* sinks, int64_t k_ld, int64_t v_ld, int gate_kind, int dtype, void* stream) {
   if (T == 0) return 0;
+  if (keep_first < 0 || chunk < 0 || (P > 0 && (keep_first > 0 || chunk > 0)))
+    return fail(-1, "lv_masked_attn: kept first tokens and chunks do not combine with pooled blocks");
+  if (sinks != nullptr) has_sink = 1;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !tok_seq || !block_tables)
     return fail(-1, "lv_window_pool_attn: null pointer");
   if (k_ld <= 0) k_ld = static_cast<int64_t>(G) * D;
@@ -308,7 +324,8 @@ int lv_window_pool_attn(const void* q, const void* k_cache, const void* v_cache,
   const int rep = H / G;
   WindowAttnParams p{q, k_cache, v_cache, kp, vp, gate, ld_gate, gate_dv, out, cu_q, ctx_lens, tok_seq, block_tables,
                      bt_stride, H, G, D, Dv, page, window, P, P > 0 ? (page + P - 1) / P : 0, scale,
-                     has_sink ? 1.0f : 0.0f, k_ld, v_ld, has_sink ? 0.0f : -1e30f};
+                     has_sink ? 1.0f : 0.0f, k_ld, v_ld, has_sink ? 0.0f : -1e30f, keep_first, chunk,
+                     static_cast<const float*>(sinks)};
   const size_t shm = sizeof(float) * (static_cast<size_t>(kMaxRep) * D + 4 * kMaxRep * kWave +
                                       4 * static_cast<size_t>(kMaxRep) * Dv + 4 * kMaxRep * 2);
   if (shm > 64 * 1024) return fail(-2, "lv_window_pool_attn: head sizes %d / %d need %zu bytes of LDS", D, Dv, shm);

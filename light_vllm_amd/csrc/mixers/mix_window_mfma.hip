@@ -35,6 +35,9 @@ struct WindowMfmaParams {
   float* ws;           // [T, H, nsplit, Dv + 4] partial read-outs, running maximum and sum
   int64_t k_ld, v_ld;  // elements between the rows of two cached tokens (G*D, G*Dv unless the caches are views of wider rows)
   float m0;            // start of the running maximum: the sink's score 0, or far below any score without a sink
+  int keep_first;      // positions below this are seen from everywhere; they take the place of the pooled tiles (P == 0)
+  int chunk;           // > 0: a query sees its own chunk of that many positions (counted from 0) up to itself; no window
+  const float* sinks;  // [H] or NULL: a learned score per query head in place of the sink's 0
 };
 
 constexpr int kTileQ = 16;
@@ -112,10 +115,13 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
   f32x4_t acc_o[DVB];
 #pragma unroll
   for (int d = 0; d < DVB; ++d) acc_o[d] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  float m = p.m0, l = split == 0 ? p.sink : 0.0f;
+  float m = p.sinks != nullptr ? p.sinks[h] : p.m0, l = split == 0 ? p.sink : 0.0f;
 
-  const int nbmax = (P > 0 && i1 - W + 1 > 0) ? (i1 - W + 1) / P : 0;      // pooled blocks the last query sees
-  const int jlo = max(0, i0 - W + 1);
+  const int chunk = p.chunk, keep = p.keep_first;
+  const int jlo = chunk > 0 ? (i0 / chunk) * chunk : max(0, i0 - W + 1);
+  const int cstart = chunk > 0 ? (pos / chunk) * chunk : 0;                // first position of this lane's query's chunk
+  // entries of the first phase: pooled blocks the last query sees, or (without a pool) kept first tokens before the token tiles
+  const int nbmax = P > 0 ? ((chunk == 0 && i1 - W + 1 > 0) ? (i1 - W + 1) / P : 0) : min(keep, jlo);
 
   // The tiles of both phases as one list: [pooled tiles | token tiles]. The V rows of the next tile and the
   // addresses of its key rows are fetched while the current tile is computed; they meet LDS behind a barrier.
@@ -125,7 +131,13 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
   const int nseg = Dv / 4;                                                // 8-byte segments of a row
 
   auto entry_rows = [&](int tile, int e, const uint16_t*& kr_, const uint16_t*& vr_) {
-    if (tile < npt) {
+    if (tile < npt && P == 0) {
+      const int ec = min(e, nbmax - 1);
+      const int pj = fdiv(ec, page, p.m_page);
+      const int64_t slot = static_cast<int64_t>(bt(pj)) * page + (ec - pj * page);
+      kr_ = p.k_cache + slot * p.k_ld + g * D;
+      vr_ = p.v_cache + slot * p.v_ld + g * Dv;
+    } else if (tile < npt) {
       const int ec = min(e, nbmax - 1);
       const int pj = fdiv(ec * P + P - 1, page, p.m_page);
       const int64_t slot = static_cast<int64_t>(bt(pj)) * p.PP + (ec - fdiv(page * pj, P, p.m_P));
@@ -244,8 +256,8 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
         for (int i = 0; i < 4; ++i) {
           const int ke = e0 + kb * 16 + 4 * lg + i;                         // the key of result row 4*lg + i
           bool vis = ke < e_end;
-          if (phase == 0) vis = vis && (ke * P + P - 1 <= pos - W);
-          else vis = vis && ke <= pos && pos - ke < W;
+          if (phase == 0) vis = vis && (P == 0 || ke * P + P - 1 <= pos - W);
+          else vis = vis && ke <= pos && ((chunk > 0 ? ke >= cstart : pos - ke < W) || ke < keep);
           s[kb][i] = vis ? acc[i] * p.scale : -INFINITY;
         }
       }
@@ -326,14 +338,15 @@ __global__ __launch_bounds__(256, (AHEAD || DVB > 8) ? 1 : 4) void window_pool_m
 // One wave per (token, query head): combines the splits' partials (each with its own running maximum), applies the gate.
 __global__ __launch_bounds__(256) void window_pool_merge_kernel(const float* __restrict__ ws, const uint16_t* __restrict__ gate,
                                                                 int64_t ld_gate, int gate_dv, uint16_t* __restrict__ out,
-                                                                int64_t items, int H, int Dv, int nsplit, float m0) {
+                                                                int64_t items, int H, int Dv, int nsplit, float m0,
+                                                                const float* __restrict__ sinks) {
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t item = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;
   if (item >= items) return;
   const int64_t t = item / H;
   const int h = static_cast<int>(item - t * H);
   const float* w = ws + item * nsplit * (Dv + 4);
-  float mm = m0;
+  float mm = sinks != nullptr ? sinks[h] : m0;
   for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, w[s * (Dv + 4) + Dv]);
   float ll = 0.0f;
   for (int s = 0; s < nsplit; ++s) ll += w[s * (Dv + 4) + Dv + 1] * expf(w[s * (Dv + 4) + Dv] - mm);
@@ -361,7 +374,21 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                                         int max_new_tokens, int H, int G, int D, int Dv, int page, int window, int P,
                                         float scale, int has_sink, int nsplit, void* workspace, int64_t T, int64_t k_ld,
                                         int64_t v_ld, int gate_kind, void* stream) {
+  return lv_masked_attn_mfma(q, k_cache, v_cache, kp, vp, gate, ld_gate, out, cu_q, ctx_lens, block_tables, bt_stride, B,
+                             max_new_tokens, H, G, D, Dv, page, window, 0, 0, P, scale, has_sink, nullptr, nsplit, workspace, T,
+                             k_ld, v_ld, gate_kind, stream);
+}
+
+extern "C" int lv_masked_attn_mfma(const void* q, const void* k_cache, const void* v_cache, const void* kp, const void* vp,
+                                   const void* gate, int64_t ld_gate, void* out, const int32_t* cu_q, const int32_t* ctx_lens,
+                                   const int32_t* block_tables, int bt_stride, int B, int max_new_tokens, int H, int G, int D,
+                                   int Dv, int page, int window, int keep_first, int chunk, int P, float scale, int has_sink,
+                                   const void* sinks, int nsplit, void* workspace, int64_t T, int64_t k_ld, int64_t v_ld,
+                                   int gate_kind, void* stream) {
   if (B == 0 || max_new_tokens <= 0) return 0;
+  if (keep_first < 0 || chunk < 0 || (P > 0 && (keep_first > 0 || chunk > 0)))
+    return fail(-1, "lv_masked_attn_mfma: kept first tokens and chunks do not combine with pooled blocks");
+  if (sinks != nullptr) has_sink = 1;
   if (!q || !k_cache || !v_cache || !out || !cu_q || !ctx_lens || !block_tables)
     return fail(-1, "lv_window_pool_attn_mfma: null pointer");
   if (P > 0 && (!kp || !vp)) return fail(-1, "lv_window_pool_attn_mfma: pooled blocks without their cache");
@@ -387,7 +414,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
                      static_cast<uint16_t*>(out), cu_q, ctx_lens, block_tables, bt_stride, H, G, D, Dv, page, window, P,
                      P > 0 ? (page + P - 1) / P : 0, ngroups, scale, has_sink ? 1.0f : 0.0f,
                      magic(page), magic(P > 0 ? P : 1), magic(Dv / 4), nsplit > 1 ? nsplit : 1, static_cast<float*>(workspace),
-                     k_ld, v_ld, m0};
+                     k_ld, v_ld, m0, keep_first, chunk, static_cast<const float*>(sinks)};
   if (nsplit > 1 && (max_new_tokens > kTileQ || workspace == nullptr || T <= 0))
     return fail(-1, "lv_window_pool_attn_mfma: key splits need one query tile per sequence and a workspace");
   const size_t shm = static_cast<size_t>(Dv) * kLdk * sizeof(uint16_t);
@@ -405,7 +432,7 @@ extern "C" int lv_window_pool_attn_mfma(const void* q, const void* k_cache, cons
     const int64_t items = T * H;
     window_pool_merge_kernel<<<dim3(static_cast<unsigned>((items + 3) / 4)), block, 0, st>>>(
         static_cast<const float*>(workspace), static_cast<const uint16_t*>(gate), ld_gate, gate_dv,
-        static_cast<uint16_t*>(out), items, H, Dv, nsplit, m0);
+        static_cast<uint16_t*>(out), items, H, Dv, nsplit, m0, static_cast<const float*>(sinks));
   }
   return launched("lv_window_pool_attn_mfma");
 }

@@ -1,6 +1,6 @@
 """SwiGLU: silu(gate) * up over the two halves of the last dim (reference "native" backend,
-lightvllm/layers/activation.py:7-29), the clamped gated unit with a sigmoid of slope alpha, and PolyNorm,
-a learned cubic of the row-normalised powers of its input."""
+lightvllm/layers/activation.py:7-29), the clamped gated unit with a sigmoid of slope alpha, PolyNorm,
+a learned cubic of the row-normalised powers of its input, and the gated unit with a choice of activation."""
 import torch
 import torch.nn.functional as F
 from torch import nn
@@ -40,3 +40,16 @@ class PolyNorm(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return mix_ops.polynorm(x, self.coef, self.eps)
+
+
+class GatedAct(nn.Module):
+    """act(gate) * up over the [gate | up] halves of the last dim; act: "gelu_tanh" (0.5 z (1 + tanh(sqrt(2/pi) (z +
+    0.044715 z^3)))), "gelu" (the exact form) or "relu2"."""
+
+    def __init__(self, act: str = "gelu_tanh"):
+        super().__init__()
+        assert act in mix_ops.ACTS
+        self.act = act
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return mix_ops.glu_act(x, self.act)

@@ -128,6 +128,8 @@ class RowParallelLinear(LinearBase):
         """reduce=False leaves this rank's partial sums: the caller reduces them together with the
         step that follows (layers.tp.all_reduce_add_rms_norm). Not with a bias, which is added once,
         after the sum."""
+        if self.tp_size == 1 and self.bias is not None:
+            return F.linear(x, self.weight, self.bias)      # one rank: the bias rides in the GEMM, one rounding
         y = F.linear(x, self.weight)
         if not reduce:
             assert self.bias is None

@@ -6,7 +6,10 @@ uses `top`, chosen by a sigmoid router.
     largest c, experts outside the `keep` highest-ranked blocks are excluded, and the `top` largest c that remain win.
     weights = s of the chosen / (their sum + 1e-20)      y = sum_chosen weight_e * W_down,e act(W_up,e h)
 
-act is the squared relu. All experts' up matrices are one [experts * ff, width] weight and all down
+act is the squared relu (or, as a choice, a gelu). Other choices of the constructor: scores by softmax over all router
+outputs instead of the sigmoid; a block ranked by its one largest c; `identity` more router outputs behind the experts'
+that stand for experts without weights, whose output is their input (they take part in scores, blocks and choice like any
+other; a token that chooses one gets weight * h from it). All experts' up matrices are one [experts * ff, width] weight and all down
 matrices one [width, experts * ff] weight. Two forms compute the same sum:
 
   * gathered (bf16, width and ff in multiples of 32, at least GATHER_FROM experts per choice): the (token,
@@ -53,25 +56,31 @@ MOE_KERNEL = "auto"   # "auto" | "masked" | "gathered" | "sorted" (tests force o
 class SparseMoE(nn.Module):
 
     def __init__(self, width: int, ff: int, experts: int, top: int, groups: int = 1, keep: int = 1,
-                 share: "SparseMoE | None" = None):
+                 share: "SparseMoE | None" = None, score: str = "sigmoid", group_rank: str = "top2", act: str = "relu2",
+                 identity: int = 0, logits_kernel: bool = False):
         super().__init__()
         assert tp_size() == 1, "the mixture of experts is not sharded: run it with tensor_parallel_size 1"
-        assert 1 <= top <= experts and groups >= 1 and experts % groups == 0 and 1 <= keep <= groups
+        routed = experts + identity                  # outputs of the router
+        assert 1 <= top <= routed and groups >= 1 and routed % groups == 0 and 1 <= keep <= groups and identity >= 0
+        assert score in ("sigmoid", "softmax") and group_rank in ("top2", "max") and act in mix_ops.ACTS
         self.width, self.ff, self.E, self.top, self.groups, self.keep = width, ff, experts, top, groups, keep
+        self.score, self.group_rank, self.act, self.identity, self.logits_kernel = score, group_rank, act, identity, logits_kernel
         if share is None:
             f32 = dict(dtype=torch.float32)
-            self.router_weight = nn.Parameter(torch.empty(experts, width, **f32))
-            self.correction = nn.Parameter(torch.zeros(experts, **f32))
+            self.router_weight = nn.Parameter(torch.empty(routed, width, **f32))
+            self.correction = nn.Parameter(torch.zeros(routed, **f32))
             self.up_weight = nn.Parameter(torch.empty(experts * ff, width))
             self.down_weight = nn.Parameter(torch.empty(width, experts * ff))
         else:
-            assert (share.width, share.ff, share.E) == (width, ff, experts)
+            assert (share.width, share.ff, share.E, share.identity) == (width, ff, experts, identity)
             self.router_weight, self.correction = share.router_weight, share.correction
             self.up_weight, self.down_weight = share.up_weight, share.down_weight
 
     def route(self, h: torch.Tensor):
-        logits = F.linear(h.float(), self.router_weight)
-        return mix_ops.moe_route(logits, self.correction, self.top, self.groups, self.keep)
+        # logits_kernel: small steps form their f32 logits straight from the activations (no widened copy)
+        logits = mix_ops.router_logits(h, self.router_weight) if self.logits_kernel else F.linear(h.float(), self.router_weight)
+        return mix_ops.moe_route(logits, self.correction, self.top, self.groups, self.keep, score=self.score,
+                                 group_rank=self.group_rank)
 
     def form(self, h: torch.Tensor) -> str:
         if MOE_KERNEL != "auto":
@@ -86,11 +95,16 @@ class SparseMoE(nn.Module):
         ids, weights, dense = self.route(h)
         form = self.form(h)
         if form == "gathered":
-            return mix_ops.moe_grouped_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff)
+            return mix_ops.moe_grouped_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff, self.act,
+                                          self.identity)
         if form == "sorted":
-            return mix_ops.moe_sorted_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff)
+            return mix_ops.moe_sorted_ff(h, ids, weights, self.up_weight, self.down_weight, self.E, self.ff, self.act,
+                                         self.identity)
         up = F.linear(h, self.up_weight)
-        return F.linear(mix_ops.relu2_scale(up, dense, self.E, self.ff), self.down_weight)
+        if self.act == "relu2" and not self.identity:
+            return F.linear(mix_ops.relu2_scale(up, dense, self.E, self.ff), self.down_weight)
+        y = F.linear(mix_ops.expert_act_scale(up, dense, self.E, self.ff, self.act), self.down_weight)
+        return mix_ops.scaled_row_add(y, h, dense[:, self.E:])      # experts without weights hand h through
 
 
 class GLUSparseMoE(nn.Module):

@@ -395,11 +395,15 @@ def pool_update(k_cache, v_cache, kp, vp, step, G, D, Dv, P):
 
 
 def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, window, P, scale, has_sink=True,
-                          gate_per_head=False):
+                          gate_per_head=False, keep_first=0, chunk=0, sinks=None):
     """Query at position i attends to cached positions j with 0 <= i - j < window and to the pooled
     entry of every block b with b*P + P - 1 <= i - window, one softmax over both, `has_sink` adding 1
     to its denominator; the result is multiplied by sigmoid(gate) when a gate is given (gate rows hold
     H*Dv numbers, one per output channel, or H with `gate_per_head`).
+    keep_first > 0: positions j < keep_first are seen from everywhere as well. chunk > 0: instead of a window, a
+    query sees the positions of its own chunk, floor(i / chunk) == floor(j / chunk), j <= i (chunks count from
+    position 0 of the sequence). sinks f32 [H]: the denominator of head h holds exp(sinks[h]) instead of 1.
+    Neither combines with pooled blocks.
     q [T, H*D] contiguous act; returns act [T, H*Dv]. k_cache and v_cache [pages, page, G, D|Dv] may be
     views of wider token rows (one cache row serving as key and, in part, as value). A window that no
     sequence reaches, no pool and no sink give plain causal softmax attention."""
@@ -407,6 +411,11 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
     page = k_cache.size(1)
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
     k_ld, v_ld = k_cache.stride(1), v_cache.stride(1)
+    assert P == 0 or (keep_first == 0 and chunk == 0)
+    if sinks is not None:
+        _f32(sinks)
+        assert sinks.numel() == H
+        has_sink = True
     if q.is_cuda:
         assert q.is_contiguous() and (gate is None or (gate.stride(1) == 1 and gate.size(1) == (H if gate_per_head else H * Dv)))
         for c, ld, d in ((k_cache, k_ld, D), (v_cache, v_ld, Dv)):
@@ -421,25 +430,27 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
             B = len(step.host_lens_q)
             if max(step.host_lens_q) <= 16:
                 most = max(c + n for c, n in zip(step.host_ctx_lens, step.host_lens_q))
-                tiles = -(-min(most, window + 16) // 64) + (-(-(max(most - window, 0) // P) // 64) if P > 0 else 0)
+                span = min(most, chunk + 16) if chunk > 0 else min(most, window + 16 + keep_first)
+                tiles = -(-span // 64) + (-(-(max(most - window, 0) // P) // 64) if P > 0 else 0)
                 nsplit = max(1, min(tiles, 256 // max(B * G * -(-(H // G) // 4), 1), 32))      # one workgroup a CU: more splits cost more in the merge than they gain (measured)
                 if nsplit > 1:
                     ws = torch.empty(T * H * nsplit * (Dv + 4), dtype=torch.float32, device=q.device)
-            _mixlib.check(lib.lv_window_pool_attn_mfma(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
-                                                       gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
-                                                       _p(step.ctx_lens), _p(step.block_tables),
-                                                       step.block_tables.stride(0), len(step.host_lens_q),
-                                                       max(step.host_lens_q), H, G, D, Dv, page, window, P, scale,
-                                                       int(has_sink), nsplit, _p(ws), T, k_ld, v_ld, 0 if gate_per_head else 1,
-                                                       _stream(q)),
-                          "lv_window_pool_attn_mfma")
+            _mixlib.check(lib.lv_masked_attn_mfma(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
+                                                  gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
+                                                  _p(step.ctx_lens), _p(step.block_tables),
+                                                  step.block_tables.stride(0), len(step.host_lens_q),
+                                                  max(step.host_lens_q), H, G, D, Dv, page, window, keep_first, chunk, P, scale,
+                                                  int(has_sink), _p(sinks), nsplit, _p(ws), T, k_ld, v_ld,
+                                                  0 if gate_per_head else 1, _stream(q)),
+                          "lv_masked_attn_mfma")
             return out
-        _mixlib.check(lib.lv_window_pool_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
-                                              gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
-                                              _p(step.ctx_lens), _p(step.tok_seq), _p(step.block_tables),
-                                              step.block_tables.stride(0), T, H, G, D, Dv, page, window, P, scale,
-                                              int(has_sink), k_ld, v_ld, 0 if gate_per_head else 1, _DT[q.dtype], _stream(q)),
-                      "lv_window_pool_attn")
+        _mixlib.check(lib.lv_masked_attn(_p(q), _p(k_cache), _p(v_cache), _p(kp), _p(vp), _p(gate),
+                                         gate.stride(0) if gate is not None else 0, _p(out), _p(step.cu_q),
+                                         _p(step.ctx_lens), _p(step.tok_seq), _p(step.block_tables),
+                                         step.block_tables.stride(0), T, H, G, D, Dv, page, window, keep_first, chunk, P, scale,
+                                         int(has_sink), _p(sinks), k_ld, v_ld, 0 if gate_per_head else 1, _DT[q.dtype],
+                                         _stream(q)),
+                      "lv_masked_attn")
         return out
     PP = pooled_slots(page, P)
     rep = H // G
@@ -450,7 +461,8 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
         for r in range(n):
             i = ctx + r
             nb = max(0, (i - window + 1) // P) if P > 0 else 0
-            rows = [_token_slot(bt, j, page) for j in range(max(0, i - window + 1), i + 1)]
+            j0 = (i // chunk) * chunk if chunk > 0 else max(0, i - window + 1)
+            rows = [_token_slot(bt, j, page) for j in list(range(min(keep_first, j0))) + list(range(j0, i + 1))]
             K, V = kc[rows].float(), vc[rows].float()
             if nb:
                 prow = [_pool_slot(bt, blk, page, P, PP) for blk in range(nb)]
@@ -459,10 +471,11 @@ def window_pool_attention(q, k_cache, v_cache, kp, vp, gate, step, H, G, D, Dv, 
             qi = q[q0 + r].float().view(G, rep, D)
             s = torch.einsum("grd,ngd->grn", qi, K) * scale
             m = s.max(-1, keepdim=True).values
+            sk = sinks.view(G, rep, 1) if sinks is not None else torch.zeros(G, rep, 1)
             if has_sink:
-                m = m.clamp(min=0)
+                m = torch.maximum(m, sk)
             e = torch.exp(s - m)
-            w = e / (e.sum(-1, keepdim=True) + (torch.exp(-m) if has_sink else 0))
+            w = e / (e.sum(-1, keepdim=True) + (torch.exp(sk - m) if has_sink else 0))
             o = torch.einsum("grn,ngv->grv", w, V).reshape(H * Dv)
             if gate is not None:
                 gr = torch.sigmoid(gate[q0 + r].float())
@@ -489,13 +502,18 @@ def rotary_inv_freq(dims: int, base: float, device, scaling: dict | None = None)
     return f.float().to(device)
 
 
-def _rotate(x, pos, inv_freq, dims):
-    """x f32 [n, ..., d]: the first `dims` entries rotated pairwise (i, i + dims/2) by pos * inv_freq[i]."""
+def _rotate(x, pos, inv_freq, dims, interleaved=False):
+    """x f32 [n, ..., d]: the first `dims` entries rotated pairwise by pos * inv_freq[i]; pair i is (i, i + dims/2),
+    or (2i, 2i + 1) with `interleaved`."""
     if dims == 0:
         return x
     half = dims // 2
     ang = pos.float().view(-1, *([1] * (x.dim() - 1))) * inv_freq.view(*([1] * (x.dim() - 1)), half)
     c, s = torch.cos(ang), torch.sin(ang)
+    if interleaved:
+        u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+        turned = torch.stack([u * c - v * s, v * c + u * s], -1).flatten(-2)
+        return torch.cat([turned, x[..., dims:]], -1)
     u, v = x[..., :half], x[..., half:dims]
     return torch.cat([u * c - v * s, v * c + u * s, x[..., dims:]], -1)
 
@@ -504,11 +522,13 @@ def _positions(step, device):
     return torch.cat([torch.arange(c, c + n, device=device) for n, c in zip(step.host_lens_q, step.host_ctx_lens)])
 
 
-def rotary_store(proj, off_q, off_k, off_v, inv_freq, head_scale, k_cache, v_cache, step, H, G, D, Dv, rot_dims):
+def rotary_store(proj, off_q, off_k, off_v, inv_freq, head_scale, k_cache, v_cache, step, H, G, D, Dv, rot_dims,
+                 interleaved=False, unit_eps=None):
     """proj act [T, ld]: queries at column off_q (H heads of D), keys at off_k (G heads of D), values at off_v
     (G heads of Dv). The first rot_dims entries of every query and key head are rotated (entry i pairs with
-    i + rot_dims/2, angle = position * inv_freq[i], f32); each query head is then multiplied by head_scale[h]
-    (f32 [H], may be None). Rotated keys and the values go to the token's row of the paged caches
+    i + rot_dims/2, or with `interleaved` entry 2i with 2i + 1; angle = position * inv_freq[i], f32); each query head is
+    then multiplied by head_scale[h] (f32 [H], may be None). With unit_eps (a number) every query and key head is first
+    divided by sqrt(mean(head^2) + unit_eps). Rotated keys and the values go to the token's row of the paged caches
     [pages, page, G, D|Dv]. Returns the queries, act [T, H*D]."""
     T = proj.size(0)
     page = k_cache.size(1)
@@ -519,17 +539,28 @@ def rotary_store(proj, off_q, off_k, off_v, inv_freq, head_scale, k_cache, v_cac
     if proj.is_cuda:
         assert proj.stride(1) == 1
         lib = _mixlib.load()
+        if interleaved or unit_eps is not None:
+            _mixlib.check(lib.lv_qk_prep_store(_p(proj), proj.stride(0), off_q, off_k, off_v, _p(inv_freq), _p(head_scale),
+                                               _p(q_out), _p(k_cache), _p(v_cache), _p(step.cu_q), _p(step.ctx_lens),
+                                               _p(step.tok_seq), _p(step.block_tables), step.block_tables.stride(0), T, H, G, D,
+                                               Dv, rot_dims, int(interleaved), int(unit_eps is not None),
+                                               float(unit_eps or 0.0), page, _DT[proj.dtype], _stream(proj)), "lv_qk_prep_store")
+            return q_out
         _mixlib.check(lib.lv_rotary_store(_p(proj), proj.stride(0), off_q, off_k, off_v, _p(inv_freq), _p(head_scale), _p(q_out),
                                           _p(k_cache), _p(v_cache), _p(step.cu_q), _p(step.ctx_lens), _p(step.tok_seq),
                                           _p(step.block_tables), step.block_tables.stride(0), T, H, G, D, Dv, rot_dims, page,
                                           _DT[proj.dtype], _stream(proj)), "lv_rotary_store")
         return q_out
     pos = _positions(step, proj.device)
-    q = _rotate(proj[:, off_q:off_q + H * D].float().view(T, H, D), pos, inv_freq, rot_dims)
+    q, k = proj[:, off_q:off_q + H * D].float().view(T, H, D), proj[:, off_k:off_k + G * D].float().view(T, G, D)
+    if unit_eps is not None:
+        q = q / torch.sqrt(q.pow(2).mean(-1, keepdim=True) + unit_eps)
+        k = k / torch.sqrt(k.pow(2).mean(-1, keepdim=True) + unit_eps)
+    q = _rotate(q, pos, inv_freq, rot_dims, interleaved)
     if head_scale is not None:
         q = q * head_scale.view(1, H, 1)
     q_out.copy_(q.reshape(T, H * D))
-    k = _rotate(proj[:, off_k:off_k + G * D].float().view(T, G, D), pos, inv_freq, rot_dims).reshape(T, G * D).to(k_cache.dtype)
+    k = _rotate(k, pos, inv_freq, rot_dims, interleaved).reshape(T, G * D).to(k_cache.dtype)
     v = proj[:, off_v:off_v + G * Dv]
     kc, vc = k_cache.view(-1, G * D), v_cache.view(-1, G * Dv)
     q0 = 0
@@ -616,10 +647,11 @@ def latent_out_gate(o, gate, per_channel: bool):
 
 
 # ------------------------------------------------------------------------------ mixture of experts
-def moe_route(logits, correction, top, groups=1, keep=1, normalize=True):
+def moe_route(logits, correction, top, groups=1, keep=1, normalize=True, score="sigmoid", group_rank="top2"):
     """logits f32 [T, E] -> (ids int32 [T, top], weights f32 [T, top], dense f32 [T, E]).
-    Scores s = sigmoid(logits); the choice goes by s + correction; with `groups` > 1 only experts of the
-    `keep` blocks of consecutive experts ranked highest by the sum of their two top selection scores stay in the selection; weights are the
+    Scores s = sigmoid(logits), or with score="softmax" the softmax over the row; the choice goes by s + correction; with
+    `groups` > 1 only experts of the `keep` blocks of consecutive experts ranked highest by the sum of their two top selection
+    scores (group_rank="max": by their top selection score) stay in the selection; weights are the
     chosen s over their sum (+ 1e-20), or the chosen s themselves without `normalize`; dense holds them at the
     chosen experts and 0 elsewhere. correction may be None."""
     T, E = logits.shape
@@ -630,14 +662,15 @@ def moe_route(logits, correction, top, groups=1, keep=1, normalize=True):
     dense = torch.empty(T, E, dtype=torch.float32, device=dev)
     if logits.is_cuda:
         lib = _mixlib.load()
-        _mixlib.check(lib.lv_moe_route(_p(logits), _p(correction), _p(ids), _p(w), _p(dense), T, E, top, groups, keep,
-                                       int(normalize), _stream(logits)), "lv_moe_route")
+        _mixlib.check(lib.lv_moe_route_scored(_p(logits), _p(correction), _p(ids), _p(w), _p(dense), T, E, top, groups, keep,
+                                              int(normalize), {"sigmoid": 0, "softmax": 1}[score],
+                                              {"top2": 0, "max": 1}[group_rank], _stream(logits)), "lv_moe_route")
         return ids, w, dense
-    s = torch.sigmoid(logits)
+    s = torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, -1)
     c = s + correction if correction is not None else s.clone()
     if groups > 1 and keep < groups:
         cg = c.view(T, groups, E // groups)
-        gs = cg.topk(min(2, E // groups), -1).values.sum(-1)
+        gs = cg.topk(min(2 if group_rank == "top2" else 1, E // groups), -1).values.sum(-1)
         best = gs.topk(keep, -1).indices
         kept = torch.zeros(T, groups, dtype=torch.bool).scatter_(1, best, True)
         c = cg.masked_fill(~kept[:, :, None], float("-inf")).reshape(T, E)
@@ -689,10 +722,64 @@ def moe_grouped_ok(h, Fe) -> bool:
     return h.dtype == torch.bfloat16 and h.size(1) % 32 == 0 and Fe % 32 == 0
 
 
-def moe_grouped_ff(h, ids, weights, up_w, down_w, E, Fe):
-    """y[t] = sum_k weights[t, k] * W_down,e relu(W_up,e h[t])^2 with e = ids[t, k], computed expert by expert on rows
+ACTS = {"relu2": 0, "gelu": 1, "gelu_tanh": 2}
+
+
+def _act(x, act):
+    """x f32 -> relu(x)^2, exact gelu, or the tanh form of gelu."""
+    if act == "relu2":
+        return torch.relu(x).pow(2)
+    return F.gelu(x, approximate="tanh" if act == "gelu_tanh" else "none")
+
+
+def glu_act(x, act="gelu_tanh"):
+    """x act [T, 2F] = [gate | up] (row stride free) -> act [T, F] = act(gate) * up."""
+    T, F2 = x.shape
+    Fh = F2 // 2
+    out = torch.empty(T, Fh, dtype=x.dtype, device=x.device)
+    if x.is_cuda:
+        assert x.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_glu_act(_p(x), x.stride(0), _p(out), T, Fh, ACTS[act], _DT[x.dtype], _stream(x)), "lv_glu_act")
+        return out
+    out.copy_(_act(x[:, :Fh].float(), act) * x[:, Fh:].float())
+    return out
+
+
+def expert_act_scale(up, dense, E, Fe, act="relu2"):
+    """up act [T, E*Fe] (all experts' up projections), dense f32 [T, >= E] (row stride free) -> act(up) * dense[t, e], act."""
+    T = up.size(0)
+    out = torch.empty_like(up)
+    if up.is_cuda:
+        assert up.is_contiguous() and dense.stride(1) == 1 and dense.dtype == torch.float32 and dense.size(1) >= E
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_expert_act_scale(_p(up), _p(dense), dense.stride(0), _p(out), T, E, Fe, ACTS[act], _DT[up.dtype],
+                                              _stream(up)), "lv_expert_act_scale")
+        return out
+    out.copy_((_act(up.float(), act).view(T, E, Fe) * dense[:, :E, None]).reshape(T, E * Fe))
+    return out
+
+
+def scaled_row_add(y, h, factors):
+    """y act [T, W] += (sum of factors[t, :]) * h[t], in place; factors f32 [T, n] (row stride free)."""
+    T, W = y.shape
+    if factors.size(1) == 0:
+        return y
+    if y.is_cuda:
+        assert y.is_contiguous() and h.is_contiguous() and h.dtype == y.dtype and factors.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_scaled_row_add(_p(y), _p(h), _p(factors), factors.stride(0), factors.size(1), T, W, _DT[y.dtype],
+                                            _stream(y)), "lv_scaled_row_add")
+        return y
+    y.copy_(y.float() + factors.sum(-1, keepdim=True) * h.float())
+    return y
+
+
+def moe_grouped_ff(h, ids, weights, up_w, down_w, E, Fe, act="relu2", n_through=0):
+    """y[t] = sum_k weights[t, k] * W_down,e act(W_up,e h[t]) with e = ids[t, k], computed expert by expert on rows
     sorted by expert: up_w [E*Fe, W], down_w [W, E*Fe]. The expert outputs are rounded to the activation dtype
-    before the weighted sum, which is in f32. Returns act [T, W]."""
+    before the weighted sum, which is in f32. A choice e >= E (at most E + n_through - 1) stands for an expert without
+    weights that hands h[t] through. Returns act [T, W]."""
     T, W = h.shape
     top = ids.size(1)
     out = torch.empty(T, W, dtype=h.dtype, device=h.device)
@@ -700,17 +787,20 @@ def moe_grouped_ff(h, ids, weights, up_w, down_w, E, Fe):
         assert moe_grouped_ok(h, Fe) and h.is_contiguous() and up_w.is_contiguous() and down_w.is_contiguous()
         assert ids.dtype == torch.int32 and ids.is_contiguous() and weights.is_contiguous() and weights.dtype == torch.float32
         lib = _mixlib.load()
-        ws = torch.empty(lib.lv_moe_grouped_workspace_bytes(T, W, Fe, E, top), dtype=torch.uint8, device=h.device)
-        _mixlib.check(lib.lv_moe_grouped_ff(_p(h), _p(ids), _p(weights), _p(up_w), _p(down_w), _p(out), _p(ws), T, W, Fe, E, top,
-                                            _stream(h)), "lv_moe_grouped_ff")
+        ws = torch.empty(lib.lv_moe_grouped_workspace_bytes(T, W, Fe, E + n_through, top), dtype=torch.uint8, device=h.device)
+        _mixlib.check(lib.lv_moe_grouped_act_ff(_p(h), _p(ids), _p(weights), _p(up_w), _p(down_w), _p(out), _p(ws), T, W, Fe, E,
+                                                n_through, top, ACTS[act], _stream(h)), "lv_moe_grouped_act_ff")
         return out
     acc = torch.zeros(T, W)
-    for e in range(E):
+    for e in range(E + n_through):
         t_idx, k_idx = (ids == e).nonzero(as_tuple=True)
         if t_idx.numel() == 0:
             continue
-        a = torch.relu(F.linear(h[t_idx], up_w[e * Fe:(e + 1) * Fe]).float()).pow(2).to(h.dtype)
-        y = F.linear(a, down_w[:, e * Fe:(e + 1) * Fe]).float()
+        if e >= E:
+            y = h[t_idx].float()
+        else:
+            a = _act(F.linear(h[t_idx], up_w[e * Fe:(e + 1) * Fe]).float(), act).to(h.dtype)
+            y = F.linear(a, down_w[:, e * Fe:(e + 1) * Fe]).float()
         acc.index_add_(0, t_idx, y * weights[t_idx, k_idx][:, None])
     out.copy_(acc)
     return out
@@ -772,19 +862,24 @@ def moe_sort(ids, E, align=1):
     return sorted_pair, inv.view_as(ids), offsets.to(torch.int32)
 
 
-def moe_combine(rows, inv, weights=None):
+def moe_combine(rows, inv, weights=None, ids=None, n_real=0, h=None):
     """rows act [M, W] (expert outputs in sorted order) -> act [T, W] = sum_k weights[t, k] * rows[inv[t, k]], in f32
-    (weights None: the plain sum)."""
+    (weights None: the plain sum). With ids [T, top], n_real and h [T, W]: a choice with ids[t, k] >= n_real takes h[t]
+    in place of its row."""
     T, top = inv.shape
     W = rows.size(1)
     out = torch.empty(T, W, dtype=rows.dtype, device=rows.device)
     if rows.is_cuda:
         assert rows.dtype == torch.bfloat16 and rows.is_contiguous() and W % 4 == 0
         assert weights is None or (weights.dtype == torch.float32 and weights.is_contiguous())
+        assert ids is None or (ids.dtype == torch.int32 and ids.is_contiguous() and h.is_contiguous() and h.dtype == rows.dtype)
         lib = _mixlib.load()
-        _mixlib.check(lib.lv_moe_combine(_p(rows), _p(inv), _p(weights), _p(out), T, W, top, _stream(rows)), "lv_moe_combine")
+        _mixlib.check(lib.lv_moe_combine_through(_p(rows), _p(inv), _p(weights), _p(out), T, W, top, _p(ids), n_real, _p(h),
+                                                 _stream(rows)), "lv_moe_combine")
         return out
     picked = rows[inv.long()].float()
+    if ids is not None:
+        picked = torch.where((ids >= n_real)[:, :, None], h.float()[:, None, :], picked)
     out.copy_((picked * weights[:, :, None] if weights is not None else picked).sum(1))
     return out
 
@@ -792,7 +887,7 @@ def moe_combine(rows, inv, weights=None):
 SORTED_ALIGN = 128
 
 
-def moe_sorted_ff(h, ids, weights, up_w, down_w, E, Fe):
+def moe_sorted_ff(h, ids, weights, up_w, down_w, E, Fe, act="relu2", n_through=0):
     """The same sum as moe_grouped_ff for large eager steps: rows sorted by expert on the device, the experts' row
     counts read back once, and each expert's two products run as vendor GEMMs on its slice of the sorted rows. One host
     synchronisation per call, so not for steps that are captured into a graph. Every expert's slice is padded to a
@@ -800,18 +895,23 @@ def moe_sorted_ff(h, ids, weights, up_w, down_w, E, Fe):
     shapes instead of a new one per expert and step, each of which would cost it a kernel selection on the host."""
     T, W = h.shape
     top = ids.size(1)
-    sorted_pair, inv, offsets = moe_sort(ids, E, SORTED_ALIGN)
+    sorted_pair, inv, offsets = moe_sort(ids, E + n_through, SORTED_ALIGN)
     off = offsets.tolist()
     xs = h.index_select(0, torch.div(sorted_pair[:off[E]], top, rounding_mode="floor"))
-    act = torch.empty(off[E], Fe, dtype=h.dtype, device=h.device)
+    mid = torch.empty(off[E], Fe, dtype=h.dtype, device=h.device)
     for e in range(E):
         if off[e + 1] > off[e]:
-            torch.mm(xs[off[e]:off[e + 1]], up_w[e * Fe:(e + 1) * Fe].t(), out=act[off[e]:off[e + 1]])
-    act.relu_().square_()
-    rows = torch.empty(off[E], W, dtype=h.dtype, device=h.device)
+            torch.mm(xs[off[e]:off[e + 1]], up_w[e * Fe:(e + 1) * Fe].t(), out=mid[off[e]:off[e + 1]])
+    if act == "relu2":
+        mid.relu_().square_()
+    else:
+        mid = F.gelu(mid, approximate="tanh" if act == "gelu_tanh" else "none")
+    rows = torch.empty(max(off[E], 1), W, dtype=h.dtype, device=h.device)    # rows of experts that hand through stay unread
     for e in range(E):
         if off[e + 1] > off[e]:
-            torch.mm(act[off[e]:off[e + 1]], down_w[:, e * Fe:(e + 1) * Fe].t(), out=rows[off[e]:off[e + 1]])
+            torch.mm(mid[off[e]:off[e + 1]], down_w[:, e * Fe:(e + 1) * Fe].t(), out=rows[off[e]:off[e + 1]])
+    if n_through:
+        return moe_combine(rows, inv.clamp(max=rows.size(0) - 1), weights, ids, E, h)
     return moe_combine(rows, inv, weights)
 
 
@@ -837,3 +937,75 @@ def moe_sorted_glu_ff(h, ids, weights, up_w, down_w, E, Fe, limit, alpha):
         if off[e + 1] > off[e]:
             torch.mm(act[off[e]:off[e + 1]], down_w[:, e * Fe:(e + 1) * Fe].t(), out=rows[off[e]:off[e + 1]])
     return moe_combine(rows, inv, None)
+
+
+# --------------------------------------------------------------------- tanh norm, two mixers side by side
+def residual_dyt(x, y1=None, y2=None, post_w1=None, post_w2=None, pair_scale=1.0, eps=1e-6, alpha=None, w=None, b=None,
+                 act_dtype=None):
+    """x [T, W] f32 (the one residual), in place:
+        post_w1 is None:  x += y1 + y2                                                   (either may be None)
+        else:             x += pair_scale * (y1 / rms(y1) * post_w1 + y2 / rms(y2) * post_w2),  rms(y) = sqrt(mean(y^2) + eps)
+    and returns the dynamic-tanh norm tanh(alpha * x) * w + b in act dtype (alpha f32 [1] or [], w and b f32 [W]), or None
+    when w is None. All arithmetic f32."""
+    T, W = x.shape
+    _f32(x, post_w1, post_w2, alpha, w, b)
+    ys = [y for y in (y1, y2) if y is not None]
+    act_dtype = act_dtype or (ys[0].dtype if ys else torch.bfloat16)
+    assert post_w1 is None or (y1 is not None and (post_w2 is not None) == (y2 is not None))
+    assert post_w1 is not None or post_w2 is None
+    out = torch.empty(T, W, dtype=act_dtype, device=x.device) if w is not None else None
+    if x.is_cuda:
+        for y in ys:
+            assert y.is_contiguous() and y.dtype == act_dtype and y.shape == (T, W)
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_residual_dyt(_p(x), _p(y1), _p(post_w1), _p(y2), _p(post_w2), pair_scale, eps, _p(alpha), _p(w),
+                                          _p(b), _p(out), T, W, _DT[act_dtype], _stream(x)), "lv_residual_dyt")
+        return out
+    if post_w1 is not None:
+        def normed(y, pw):
+            yf = y.float()
+            return yf / torch.sqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * pw
+        add = normed(y1, post_w1)
+        if y2 is not None:
+            add = add + normed(y2, post_w2)
+        x.add_(pair_scale * add)
+    else:
+        for y in ys:
+            x.add_(y.float())
+    if w is None:
+        return None
+    out.copy_(torch.tanh(alpha * x) * w + b)
+    return out
+
+
+# ------------------------------------------------------------------------------- lightning attention
+def lightning_attention(proj, off_q, off_k, off_v, decay, state, step, H, D, Dv):
+    """Linear attention with a constant decay per head. proj act [T, ld]: H query heads of D at column off_q, H key heads of
+    D at off_k, H value heads of Dv at off_v; q, k, v = silu of those columns. Per head and token
+        S <- decay[h] * S + k v^T;   o = S^T q
+    state f32 [slots, H, D, Dv] (taken as zero for a sequence with no context), updated in place; decay f32 [H].
+    Returns o f32 [T, H, Dv]."""
+    T = proj.size(0)
+    _f32(decay, state)
+    assert state.shape[1:] == (H, D, Dv) and decay.numel() == H
+    o = torch.empty(T, H, Dv, dtype=torch.float32, device=proj.device)
+    if proj.is_cuda:
+        assert proj.stride(1) == 1
+        lib = _mixlib.load()
+        _mixlib.check(lib.lv_lightning_attn(_p(proj), proj.stride(0), off_q, off_k, off_v, _p(decay), _p(state), _p(step.cu_q),
+                                            _p(step.ctx_lens), _p(step.slots), _p(o), len(step.host_lens_q), H, D, Dv,
+                                            _DT[proj.dtype], _stream(proj)), "lv_lightning_attn")
+        return o
+    q = F.silu(proj[:, off_q:off_q + H * D].float()).view(T, H, D)
+    k = F.silu(proj[:, off_k:off_k + H * D].float()).view(T, H, D)
+    v = F.silu(proj[:, off_v:off_v + H * Dv].float()).view(T, H, Dv)
+    q0 = 0
+    for b, (n, ctx) in enumerate(zip(step.host_lens_q, step.host_ctx_lens)):
+        slot = step.host_slots[b]
+        S = state[slot].clone() if ctx > 0 else torch.zeros(H, D, Dv)
+        for t in range(q0, q0 + n):
+            S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S
+        q0 += n
+    return o

@@ -31,11 +31,17 @@ def _givozen():
     return GivozenForCausalLM
 
 
+def _bisuzen():
+    from .bisuzen import BisuzenForCausalLM
+    return BisuzenForCausalLM
+
+
 MODELS = {
     "Qwen3ForCausalLM": _qwen3,
     "Kagalorn": _kagalorn,
     "Bokulorn": _bokulorn,
     "Givozen": _givozen,
+    "Bisuzen": _bisuzen,
 }
 DEFAULT = "Qwen3ForCausalLM"
 
