@@ -285,7 +285,7 @@ def random_weights(cfg, seed: int) -> dict:
     out = {}
     for name, shape in tensor_shapes(cfg).items():
         leaf = name.rsplit(".", 1)[-1]
-        x = torch.randn(*shape, generator=g)
+        x = torch.randn(tuple(shape), generator=g)
         if leaf == "alpha":
             x = 0.8 + 0.2 * x
         elif leaf == "b":
