@@ -1042,6 +1042,199 @@ def givozen_leg(sizes, batch, prompt_len, new_tokens):
     print(json.dumps(out), flush=True)
 
 
+# --mixers-design bisuzen: the Bisuzen design (layers whose mixer is a windowed attention with kept first tokens and learned
+# sinks beside a lightning attention, layers of chunked attention with unit-normed heads, tanh norms, gated dense and
+# softmax-routed expert feed-forwards with identity experts, a looped stretch of layers) beside Givozen, the closest existing
+# model (one f32 residual, the same paged attention kernel, dense and expert feed-forwards, looped layers), at equal width,
+# layer runs, head counts and active feed-forward parameters.
+BISUZEN_SIZES = {
+    "2k": dict(experts=30, identity=2, top=4, groups=4, keep=2, rot_dims=64, window=512, keep_first=4, chunk=512, state_heads=16),
+    "4k": dict(experts=30, identity=2, top=4, groups=4, keep=2, rot_dims=64, window=512, keep_first=4, chunk=512, state_heads=32),
+}
+
+
+def _bisuzen_config(z, sz):
+    from light_vllm_amd.models.bisuzen import BisuzenConfig
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    Hs = sz["state_heads"]
+    left = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "rot": {"base": 500000.0, "dims": sz["rot_dims"]},
+            "mask": {"size": sz["window"], "keep_first": sz["keep_first"]}}
+    right = {"heads": Hs, "dim": D, "vdim": D, "decay": [1.0 - 2.0 ** (-5.0 - 5.0 * i / max(Hs - 1, 1)) for i in range(Hs)]}
+    att = {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5, "mask": {"size": sz["chunk"]}}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // sz["top"]},
+           "router": {"experts": sz["experts"], "identity": sz["identity"], "top": sz["top"],
+                      "groups": {"count": sz["groups"], "keep": sz["keep"]}}}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    looped = 2 if z["layers"] >= 6 else 1      # layers that run twice: as many layer runs as the other model has
+    n = z["layers"] - looped
+    layers = [{"type": "parallel" if i % 2 == 0 else "attention", "mixer": {"left": left, "right": right} if i % 2 == 0 else att,
+               "mlp": dense if i == 0 else moe} for i in range(n)]
+    return BisuzenConfig.from_dict({"vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+                                    "layers": layers, "loop": {"start": 1, "stop": 1 + looped, "times": 2}})
+
+
+def _bisuzen_kernel_table(z, sz, gz, bz, dev, batch, prompt_len):
+    """Each kernel of the design alone at one layer's shapes (prompt step and decode step), beside the kernel of Givozen
+    (or, for the recurrence and the experts, of Kagalorn and Bokulorn) that does the like job."""
+    from light_vllm_amd import mix_ops
+    from light_vllm_amd.layers.moe import SparseMoE
+    from light_vllm_amd.layers.rotary_attention import NO_WINDOW
+    from light_vllm_amd.utils.context import RaggedStep
+    bf = torch.bfloat16
+    W, H, G, D, Hs = z["width"], z["heads"], z["kv_heads"], z["dim"], sz["state_heads"]
+    E, ident, top, Fe, rd = sz["experts"], sz["identity"], sz["top"], z["ff"] // sz["top"], sz["rot_dims"]
+    window, keep, chunk = sz["window"], sz["keep_first"], sz["chunk"]
+    page = 256
+    rows = []
+
+    def step_of(lens_q, ctx):
+        B = len(lens_q)
+        cu, tok = [0], []
+        for b, n_ in enumerate(lens_q):
+            cu.append(cu[-1] + n_)
+            tok += [b] * n_
+        per = -(-(max(ctx) + max(lens_q)) // page)
+        tables = [[b * per + j for j in range(per)] for b in range(B)]
+        i32 = dict(dtype=torch.int32, device=dev)
+        return RaggedStep(torch.tensor(cu, **i32), torch.tensor(ctx, **i32), torch.arange(B, **i32),
+                          torch.tensor(tok, **i32), torch.tensor(tables, **i32), lens_q, ctx, list(range(B)), tables), B * per
+
+    def add(name, phase, fn, nbytes=0, flops=0, like=None, matrix=True):
+        us = _event_time(fn, 20, 3) * 1e6
+        rec = {"kernel": name, "phase": phase, "us": round(us, 1)}
+        if nbytes:
+            rec["of_hbm_roofline"] = round(nbytes / us / 1e3 / (HBM_BPS / 1e9), 3)
+        if flops:
+            rec["TFLOPs"] = round(flops / us / 1e6, 2)
+            if matrix:
+                rec["of_mfma_roofline"] = round(flops / us / 1e6 / (MFMA_FLOPS / 1e12), 4)
+        if like:
+            rec["like"] = like
+        rows.append(rec)
+
+    old_default = torch.get_default_dtype()
+    torch.set_default_dtype(bf)
+    try:
+        moe = SparseMoE(W, Fe, E, top, sz["groups"], sz["keep"], score="softmax", group_rank="max", act="gelu", identity=ident,
+                        logits_kernel=True).to(dev)
+        bmoe = SparseMoE(W, z["ff"] // bz["top"], bz["experts"], bz["top"], bz["groups"], bz["keep"]).to(dev)
+    finally:
+        torch.set_default_dtype(old_default)
+    for prm in list(moe.parameters()) + list(bmoe.parameters()):
+        prm.data.normal_(0.0, 0.02)
+    for phase, lens_q, ctx in (("prompt", [prompt_len] * batch, [0] * batch), ("decode", [1] * batch, [prompt_len] * batch)):
+        step, pages = step_of(lens_q, ctx)
+        T = sum(lens_q)
+        x = torch.randn(T, W, device=dev)
+        y1, y2 = torch.randn(T, W, device=dev, dtype=bf), torch.randn(T, W, device=dev, dtype=bf)
+        nw, alpha = torch.ones(W, device=dev), torch.full((1,), 0.5, device=dev)
+        add("residual_dyt", phase, lambda: mix_ops.residual_dyt(x, y1, None, None, None, 1.0, 1e-6, alpha, nw, nw, bf), nbytes=T * W * 12)
+        add("residual_dyt (two normed mixer outputs)", phase,
+            lambda: mix_ops.residual_dyt(x, y1, y2, nw, nw, 0.5, 1e-6, alpha, nw, nw, bf), nbytes=T * W * 14)
+        add("givozen sandwich_add_norm", phase, lambda: mix_ops.sandwich_add_norm(x, y1, nw, None, None, nw, 1.0, 1e-6, bf),
+            nbytes=T * W * 12, like="residual_dyt")
+        # attention inputs: unit norm or rotation, cache write
+        cols = H * D + 2 * G * D
+        proj = torch.randn(T, cols + H, device=dev, dtype=bf)
+        inv_freq = mix_ops.rotary_inv_freq(rd, 500000.0, dev)
+        temp = torch.ones(H, device=dev)
+        kc = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        vc = torch.zeros(pages, page, G, D, device=dev, dtype=bf)
+        prep_bytes = T * cols * 4
+        add("qk_prep_store (pairs side by side rotated)", phase,
+            lambda: mix_ops.rotary_store(proj, 0, H * D, H * D + G * D, inv_freq, None, kc, vc, step, H, G, D, D, rd, interleaved=True),
+            nbytes=prep_bytes)
+        add("qk_prep_store (heads divided by their rms)", phase,
+            lambda: mix_ops.rotary_store(proj, 0, H * D, H * D + G * D, None, None, kc, vc, step, H, G, D, D, 0, unit_eps=1e-6),
+            nbytes=prep_bytes)
+        add("givozen rotary_store", phase,
+            lambda: mix_ops.rotary_store(proj, 0, H * D, H * D + G * D, inv_freq, temp, kc, vc, step, H, G, D, D, rd),
+            nbytes=prep_bytes, like="qk_prep_store")
+        q = mix_ops.rotary_store(proj, 0, H * D, H * D + G * D, inv_freq, None, kc, vc, step, H, G, D, D, rd, interleaved=True)
+        sinks = torch.zeros(H, device=dev)
+        gate = proj[:, cols:]
+        pos = [i for n_, c0 in zip(lens_q, ctx) for i in range(c0, c0 + n_)]
+        keys_full = sum(i + 1 for i in pos)
+        keys_win = sum(min(i + 1, window) + min(keep, max(i + 1 - window, 0)) for i in pos)
+        keys_chunk = sum(i % chunk + 1 for i in pos)
+        wattn = lambda: mix_ops.window_pool_attention(q, kc, vc, None, None, None, step, H, G, D, D, window, 0, D ** -0.5,  # noqa: E731
+                                                      has_sink=False, keep_first=keep, sinks=sinks)
+        cattn = lambda: mix_ops.window_pool_attention(q, kc, vc, None, None, None, step, H, G, D, D, NO_WINDOW, 0, D ** -0.5,  # noqa: E731
+                                                      has_sink=False, chunk=chunk)
+        gattn = lambda: mix_ops.window_pool_attention(q, kc, vc, None, None, gate, step, H, G, D, D, NO_WINDOW, 0, D ** -0.5,  # noqa: E731
+                                                      has_sink=False, gate_per_head=True)
+        if phase == "prompt":
+            add("windowed attention with kept tokens and sinks", phase, wattn, flops=keys_win * H * D * 4)
+            add("chunked attention", phase, cattn, flops=keys_chunk * H * D * 4)
+            add("givozen gated rotary attention", phase, gattn, flops=keys_full * H * D * 4, like="windowed / chunked attention")
+        else:
+            add("windowed attention with kept tokens and sinks", phase, wattn, nbytes=keys_win * G * D * 4)
+            add("chunked attention", phase, cattn, nbytes=keys_chunk * G * D * 4)
+            add("givozen gated rotary attention", phase, gattn, nbytes=keys_full * G * D * 4, like="windowed / chunked attention")
+        # the decaying state beside the delta rule
+        B = len(lens_q)
+        lproj = torch.randn(T, 4 * Hs * D, device=dev, dtype=bf)
+        decay = torch.full((Hs,), 0.99, device=dev)
+        state = torch.zeros(B, Hs, D, D, device=dev)
+        state_bytes = B * Hs * D * D * 8 + T * Hs * D * (3 * 2 + 4)
+        add("lightning_attention", phase, lambda: mix_ops.lightning_attention(lproj, 0, Hs * D, 2 * Hs * D, decay, state, step, Hs, D, D),
+            flops=T * Hs * D * D * 4, nbytes=state_bytes if phase == "decode" else 0, matrix=False)
+        qn, kn = torch.randn(T, G, D, device=dev) * D ** -0.5, torch.randn(T, G, D, device=dev) * D ** -0.5
+        dv = torch.randn(T, Hs, D, device=dev)
+        beta, dec = torch.rand(T, Hs, device=dev), torch.full((T, Hs), 0.99, device=dev)
+        dstate = torch.zeros(B, Hs, D, D, device=dev)
+        add("kagalorn gated_delta_rule", phase, lambda: mix_ops.gated_delta_rule(qn, kn, dv, beta, dec, dstate, step),
+            flops=T * Hs * D * D * 6, nbytes=(B * Hs * D * D * 8 + T * (2 * G * D + 2 * Hs * D) * 4) if phase == "decode" else 0,
+            like="lightning_attention", matrix=False)
+        o = torch.randn(T, Hs, D, device=dev)
+        gw = torch.ones(Hs * D, device=dev)
+        lgate = lproj[:, 3 * Hs * D:]
+        add("norm over all heads with gate", phase, lambda: mix_ops.head_norm_gate(o.view(T, 1, Hs * D), lgate, gw, 1e-6, bf, "sigmoid"),
+            nbytes=T * Hs * D * 8)
+        add("kagalorn norm per head with gate", phase, lambda: mix_ops.head_norm_gate(o, lgate, gw[:D], 1e-6, bf, "silu"),
+            nbytes=T * Hs * D * 8, like="norm over all heads with gate")
+        # feed-forwards
+        h = torch.randn(T, W, device=dev, dtype=bf)
+        zg = torch.randn(T, 2 * z["ff"], device=dev, dtype=bf)
+        add("glu_act (tanh gelu)", phase, lambda: mix_ops.glu_act(zg, "gelu_tanh"), nbytes=T * z["ff"] * 6)
+        add("kagalorn clamped_glu", phase, lambda: mix_ops.clamped_glu(zg, 7.0, 1.702), nbytes=T * z["ff"] * 6, like="glu_act")
+        with torch.inference_mode():
+            wg = torch.randn(2 * z["ff"], W, device=dev, dtype=bf) * 0.02
+            wd = torch.randn(W, z["ff"], device=dev, dtype=bf) * 0.02
+            add("dense gated feed-forward", phase,
+                lambda: torch.nn.functional.linear(mix_ops.glu_act(torch.nn.functional.linear(h, wg), "gelu_tanh"), wd),
+                flops=T * z["ff"] * W * 6)
+            add("kagalorn dense feed-forward", phase,
+                lambda: torch.nn.functional.linear(mix_ops.clamped_glu(torch.nn.functional.linear(h, wg), 7.0, 1.702), wd),
+                flops=T * z["ff"] * W * 6, like="dense gated feed-forward")
+            weight_bytes = min(T * top, E) * 2 * Fe * W * 2
+            bweight_bytes = min(T * bz["top"], bz["experts"]) * 2 * (z["ff"] // bz["top"]) * W * 2
+            add("expert feed-forward (softmax router to sum, identity experts)", phase, lambda: moe(h),
+                flops=T * top * Fe * W * 4, nbytes=weight_bytes if phase == "decode" else 0)
+            add("bokulorn moe feed-forward", phase, lambda: bmoe(h), flops=T * bz["top"] * (z["ff"] // bz["top"]) * W * 4,
+                nbytes=bweight_bytes if phase == "decode" else 0, like="expert feed-forward (softmax router to sum, identity experts)")
+    return rows
+
+
+def bisuzen_leg(sizes, batch, prompt_len, new_tokens):
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    out = {"metric": "mixers: Bisuzen beside Givozen at equal size", "dtype": "bf16", "data": "synthetic, random weights",
+           "batch": batch, "prompt_len": prompt_len, "new_tokens": new_tokens, "sizes": []}
+    for name in sizes:
+        z, sz, gz, bz = MIXER_SIZES[name], BISUZEN_SIZES[name], GIVOZEN_SIZES[name], BOKULORN_SIZES[name]
+        rec = {"size": name, **z, **sz}
+        cache_tokens = batch * 256 * (-(-(prompt_len + new_tokens) // 256))
+        kw = dict(kvcache_block_size=256, max_cache_tokens=cache_tokens)
+        rec["bisuzen"] = _engine_rates(_bisuzen_config(z, sz), batch, prompt_len, new_tokens, **kw)
+        rec["bisuzen_graph"] = _engine_rates(_bisuzen_config(z, sz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        rec["givozen"] = _engine_rates(_givozen_config(z, gz), batch, prompt_len, new_tokens, **kw)
+        rec["givozen_graph"] = _engine_rates(_givozen_config(z, gz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        rec["kernels"] = _bisuzen_kernel_table(z, sz, gz, bz, dev, batch, prompt_len)
+        out["sizes"].append(rec)
+    print(json.dumps(out), flush=True)
+
+
 def mixers_leg(sizes, batch, prompt_len, new_tokens):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -1113,13 +1306,15 @@ def main():
                          "(proves launcher, rendezvous, graph and JSON path; not a measurement)")
     ap.add_argument("--mixers", default="", help="comma list of sizes (2k, 4k): instead of the default workload, "
                     "run the Kagalorn design beside Qwen3 at equal size and time its kernels one by one")
-    ap.add_argument("--mixers-design", default="kagalorn", choices=("kagalorn", "bokulorn", "givozen"),
+    ap.add_argument("--mixers-design", default="kagalorn", choices=("kagalorn", "bokulorn", "givozen", "bisuzen"),
                     help="with --mixers: kagalorn (beside Qwen3), bokulorn (beside Kagalorn, its closest relative) or "
-                         "givozen (beside Bokulorn, its closest relative)")
+                         "givozen (beside Bokulorn, its closest relative) or bisuzen (beside Givozen, its closest relative)")
     ap.add_argument("--mixers-batch", type=int, default=16)
     ap.add_argument("--mixers-prompt", type=int, default=1024)
     ap.add_argument("--mixers-new", type=int, default=17)
     args = ap.parse_args()
+    if args.mixers and args.mixers_design == "bisuzen":
+        return bisuzen_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
     if args.mixers and args.mixers_design == "givozen":
         return givozen_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
     if args.mixers and args.mixers_design == "bokulorn":

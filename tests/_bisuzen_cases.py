@@ -114,10 +114,12 @@ def _paged(k, v, page, dtype, device, g):
 
 
 def case_masked_attention(device, dtype):
-    """Windows with kept first tokens and a learned sink, and chunks, over a paged cache. EVERY key scores high along one
-    direction, with a value of its own, so that one key too many or too few at an edge (window, kept tokens, chunk, page)
-    moves the result by far more than the tolerance; one head's sink is large enough to take half the weight, another's
-    small enough to vanish. Prompt-shaped, decode-shaped and portion-shaped launches."""
+    """Windows with kept first tokens and a learned sink, and chunks, over a paged cache. A few beacon keys score far
+    above the hundreds of others: the last kept token and the first one not kept, rows either side of page borders and
+    of chunk borders, one in the middle. A query that has a beacon just inside or just outside its window or chunk gives
+    a result of another order when it sees one key too many or too few; one head's sink is large enough to take most of
+    the weight where no beacon is seen, another's small enough to vanish. Prompt-shaped, decode-shaped and
+    portion-shaped launches."""
     from light_vllm_amd import mix_ops
     shapes = ((4, 2, 12, 10, 16, 150, 9, 3, 0), (1, 1, 40, 70, 64, 200, 70, 0, 0), (10, 1, 6, 4, 16, 90, 1, 5, 0),
               (5, 1, 32, 16, 16, 170, 33, 17, 0), (4, 2, 16, 48, 32, 210, 64, 1, 0), (2, 2, 48, 32, 64, 200, 41, 6, 0),
@@ -125,13 +127,17 @@ def case_masked_attention(device, dtype):
               (3, 3, 64, 64, 64, 300, 1, 0, 129), (2, 2, 16, 16, 16, 80, 1, 0, 1))
     for (H, G, D, Dv, page, L, window, keep, chunk) in shapes:
         g = torch.Generator().manual_seed(L + H)
+        beacons = {keep - 1, keep, page - 1, page, 2 * page + 1, 50} | ({chunk - 1, chunk, 2 * chunk - 1, 2 * chunk} if chunk else set())
+        beacons = sorted(j for j in beacons if 0 <= j < L)
         e = torch.zeros(D); e[D - 1] = 1.0
-        k = 0.2 * torch.randn(L, G, D, generator=g) + 2.0 * e
-        v = torch.randn(L, G, Dv, generator=g) + 0.02 * torch.arange(L).view(L, 1, 1)
-        q = 0.2 * torch.randn(L, H, D, generator=g) + 2.0 * e
+        k = 0.3 * torch.randn(L, G, D, generator=g)
+        for j in beacons:
+            k[j] += 6.0 * e
+        v = torch.randn(L, G, Dv, generator=g)
+        q = 0.3 * torch.randn(L, H, D, generator=g) + 3.0 * e
         sinks = torch.linspace(-6.0, 4.0, H) if H > 1 else torch.tensor([2.0])
         k, v, q = (t.to(_dt(dtype)).float() for t in (k, v, q))
-        scale = 0.6
+        scale = 0.7
         vis = oracle.chunk_visible(chunk) if chunk else oracle.window_visible(window, keep)
         use_sink = chunk == 0
         want = torch.cat([oracle.masked_softmax_head(q[:, h].to(F64), k[:, h // (H // G)].to(F64), v[:, h // (H // G)].to(F64), scale,
@@ -152,15 +158,19 @@ def case_masked_attention(device, dtype):
 
         every = list(range(L))
         check(run(K.make_step([L], [0], [0], [table], device), every), every, "prompt")
-        edges = {0, 1, keep - 1, keep, keep + 1, window - 1, window, window + keep, page - 1, page, 2 * page}
+        # queries beside every beacon, queries that have one at the edge of their window, queries beside chunk borders
+        near = {i for j in beacons for i in (j - 1, j, j + 1)}
         if chunk:
-            edges |= {chunk - 1, chunk, chunk + 1, 2 * chunk - 1, 2 * chunk, 2 * chunk + 1}
-        idx = sorted({i for j in edges for i in (j - 1, j, j + 1) if 0 <= i < L} | set(range(L - 12, L)))
+            near |= {c * chunk + d for c in range(1, 4) for d in (-2, -1, 0, 1)}
+        else:
+            near |= {j + window + d for j in beacons for d in (-2, -1, 0, 1)}
+        idx = sorted({i for i in near if 0 <= i < L} | set(range(L - 12, L)))
         check(run(K.make_step([1] * len(idx), idx, [0] * len(idx), [table] * len(idx), device), idx), idx, "decode")
         few = idx[-3:]
         check(run(K.make_step([1] * 3, few, [0] * 3, [table] * 3, device), few), few, "decode, few sequences")
         check(run(K.make_step([2], [L - 2], [0], [table], device), [L - 2, L - 1]), [L - 2, L - 1], "two tokens behind a long context")
-        # portions that straddle a page border, a window's or chunk's edge, beside the start of a sequence
+        # portions that straddle a page border and the edge at which the first beacons leave the window or chunk,
+        # beside the start of a sequence and the end of another
         cut = (chunk or window) + keep
         a, b = max(page - 1, 1), min(max(page + 1, cut + 2), L)
         rows = list(range(a, b)) + list(range(5)) + list(range(L - 19, L))
