@@ -1216,7 +1216,7 @@ def _bisuzen_kernel_table(z, sz, gz, bz, dev, batch, prompt_len):
     return rows
 
 
-def bisuzen_leg(sizes, batch, prompt_len, new_tokens):
+def bisuzen_leg(sizes, batch, prompt_len, new_tokens, engine_only=False):
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     out = {"metric": "mixers: Bisuzen beside Givozen at equal size", "dtype": "bf16", "data": "synthetic, random weights",
@@ -1228,6 +1228,9 @@ def bisuzen_leg(sizes, batch, prompt_len, new_tokens):
         kw = dict(kvcache_block_size=256, max_cache_tokens=cache_tokens)
         rec["bisuzen"] = _engine_rates(_bisuzen_config(z, sz), batch, prompt_len, new_tokens, **kw)
         rec["bisuzen_graph"] = _engine_rates(_bisuzen_config(z, sz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
+        if engine_only:              # a run to be profiled: this design's kernels only
+            out["sizes"].append(rec)
+            continue
         rec["givozen"] = _engine_rates(_givozen_config(z, gz), batch, prompt_len, new_tokens, **kw)
         rec["givozen_graph"] = _engine_rates(_givozen_config(z, gz), batch, prompt_len, new_tokens, enforce_eager=False, **kw)
         rec["kernels"] = _bisuzen_kernel_table(z, sz, gz, bz, dev, batch, prompt_len)
@@ -1309,12 +1312,15 @@ def main():
     ap.add_argument("--mixers-design", default="kagalorn", choices=("kagalorn", "bokulorn", "givozen", "bisuzen"),
                     help="with --mixers: kagalorn (beside Qwen3), bokulorn (beside Kagalorn, its closest relative) or "
                          "givozen (beside Bokulorn, its closest relative) or bisuzen (beside Givozen, its closest relative)")
+    ap.add_argument("--mixers-engine-only", action="store_true",
+                    help="with --mixers-design bisuzen: only that design's engine runs (eager and from graphs), for a profiler")
     ap.add_argument("--mixers-batch", type=int, default=16)
     ap.add_argument("--mixers-prompt", type=int, default=1024)
     ap.add_argument("--mixers-new", type=int, default=17)
     args = ap.parse_args()
     if args.mixers and args.mixers_design == "bisuzen":
-        return bisuzen_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
+        return bisuzen_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new,
+                           args.mixers_engine_only)
     if args.mixers and args.mixers_design == "givozen":
         return givozen_leg([x for x in args.mixers.split(",") if x], args.mixers_batch, args.mixers_prompt, args.mixers_new)
     if args.mixers and args.mixers_design == "bokulorn":

@@ -7,6 +7,7 @@
 //   qk_prep_store_kernel     one wave per head of a token: optional division of a query or key head by its root mean
 //                            square, optional rotation of the head's first entries (pairs side by side or half a
 //                            rotated part apart), a factor per query head, keys and values written to the paged caches.
+//                            A form with four entries per lane and several heads per wave serves aligned sizes.
 //   lightning_attn_kernel    S <- decay_h S + k v^T, o = S^T q per head over the new tokens of every sequence, the state
 //                            in f32 in the sequence's slot; q, k, v = silu of columns of the input projection. The four
 //                            waves own a quarter of the state's rows each and never meet inside a chunk of tokens.
@@ -170,6 +171,64 @@ __global__ __launch_bounds__(256) void qk_prep_store_kernel(QkPrepParams p) {
   const int GDv = p.G * p.Dv;
   T* v_out = static_cast<T*>(p.v_cache) + slot * GDv;
   for (int i = threadIdx.x; i < GDv; i += blockDim.x) v_out[i] = row[p.off_v + i];
+}
+
+// Four entries per lane: a head of D <= 256 entries sits in P lanes (the power of two at or above D / 4), so a wave holds
+// 64 / P heads at once, each value is read once and stays in registers between the sum of squares and the rotation, and
+// pairs that lie side by side need no second read at all. Taken when head sizes, the rotated part, column offsets and row
+// strides are multiples of four (eight for the rotated part) and the rows are aligned.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_prep_store_vec_kernel(QkPrepParams p, int P) {
+  extern __shared__ __attribute__((aligned(16))) float cs[];   // [rot_dims/2] cosines | [rot_dims/2] sines
+  const int64_t t = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int b = p.tok_seq[t];
+  const int pos = p.ctx_lens[b] + static_cast<int>(t) - p.cu_q[b];
+  const int64_t slot = static_cast<int64_t>(p.block_tables[static_cast<int64_t>(b) * p.bt_stride + pos / p.page]) * p.page + pos % p.page;
+  const int half = p.rot_dims / 2, D = p.D;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float s, c;
+    sincosf(static_cast<float>(pos) * p.inv_freq[i], &s, &c);
+    cs[i] = c;
+    cs[half + i] = s;
+  }
+  __syncthreads();
+  const T* row = static_cast<const T*>(p.proj) + t * p.ld;
+  T* q_out = static_cast<T*>(p.q_out) + t * p.H * D;
+  T* k_out = static_cast<T*>(p.k_cache) + slot * p.G * D;
+  const int per_wave = kWave / P, sub = lane / P, j = 4 * (lane % P);
+  const int heads = p.H + p.G;
+  for (int hd0 = 0; hd0 < heads; hd0 += 4 * per_wave) {          // the same trip count for every lane: the sums below shuffle
+    const int hd = hd0 + wave * per_wave + sub;
+    const bool live = hd < heads && j < D;
+    const bool is_q = hd < p.H;
+    const T* head = row + (is_q ? p.off_q + hd * D : p.off_k + (hd - p.H) * D);
+    float4 v = live ? ld4(head + j) : float4{0.0f, 0.0f, 0.0f, 0.0f};
+    float f = (live && is_q && p.head_scale != nullptr) ? p.head_scale[hd] : 1.0f;
+    if (p.unit_norm) {
+      float ss = (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+      for (int o = P >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, kWave);
+      f /= sqrtf(ss / static_cast<float>(D) + p.eps);
+    }
+    if (!live) continue;
+    if (j < p.rot_dims) {
+      if (p.interleaved) {
+        const int i = j >> 1;
+        const float c0 = cs[i], s0 = cs[half + i], c1 = cs[i + 1], s1 = cs[half + i + 1];
+        v = float4{v.x * c0 - v.y * s0, v.y * c0 + v.x * s0, v.z * c1 - v.w * s1, v.w * c1 + v.z * s1};
+      } else if (j < half) {
+        const float4 u = ld4(head + j + half), c = ld4(cs + j), sn = ld4(cs + half + j);
+        v = float4{v.x * c.x - u.x * sn.x, v.y * c.y - u.y * sn.y, v.z * c.z - u.z * sn.z, v.w * c.w - u.w * sn.w};
+      } else {
+        const float4 u = ld4(head + j - half), c = ld4(cs + j - half), sn = ld4(cs + j);
+        v = float4{v.x * c.x + u.x * sn.x, v.y * c.y + u.y * sn.y, v.z * c.z + u.z * sn.z, v.w * c.w + u.w * sn.w};
+      }
+    }
+    st4((is_q ? q_out + hd * D : k_out + (hd - p.H) * D) + j, float4{v.x * f, v.y * f, v.z * f, v.w * f});
+  }
+  const int GDv = p.G * p.Dv;
+  T* v_out = static_cast<T*>(p.v_cache) + slot * GDv;
+  for (int i = threadIdx.x * 4; i < GDv; i += blockDim.x * 4) st4(v_out + i, ld4(row + p.off_v + i));
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -374,9 +433,20 @@ int lv_qk_prep_store(const void* proj, int64_t ld, int off_q, int off_k, int off
                  q_out, k_cache, v_cache, cu_q, ctx_lens, tok_seq, block_tables, bt_stride, H, G, D, Dv, rot_dims, page,
                  interleaved != 0, unit_norm != 0, eps};
   dim3 grid(static_cast<unsigned>(T)), block(256);
-  if (dtype == LV_MIX_BF16) qk_prep_store_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(p);
-  else if (dtype == LV_MIX_F32) qk_prep_store_kernel<float><<<grid, block, shm, as_stream(stream)>>>(p);
-  else return fail(-1, "lv_qk_prep_store: dtype %d", dtype);
+  if (dtype != LV_MIX_BF16 && dtype != LV_MIX_F32) return fail(-1, "lv_qk_prep_store: dtype %d", dtype);
+  auto aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  const bool vec4 = D % 4 == 0 && D <= 4 * kWave && Dv % 4 == 0 && rot_dims % 8 == 0 && ld % 4 == 0 && off_q % 4 == 0 &&
+                    off_k % 4 == 0 && off_v % 4 == 0 && aligned(proj) && aligned(q_out) && aligned(k_cache) && aligned(v_cache);
+  if (vec4) {
+    int P = 1;
+    while (4 * P < D) P <<= 1;                       // lanes that hold one head
+    if (dtype == LV_MIX_BF16) qk_prep_store_vec_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(p, P);
+    else qk_prep_store_vec_kernel<float><<<grid, block, shm, as_stream(stream)>>>(p, P);
+  } else if (dtype == LV_MIX_BF16) {
+    qk_prep_store_kernel<bf16_t><<<grid, block, shm, as_stream(stream)>>>(p);
+  } else {
+    qk_prep_store_kernel<float><<<grid, block, shm, as_stream(stream)>>>(p);
+  }
   return launched("lv_qk_prep_store");
 }
 

@@ -53,52 +53,61 @@ def case_residual_dyt(device, dtype):
 
 
 def case_qk_prep(device, dtype):
-    """Division of every head by its root mean square and rotation of pairs (2i, 2i+1) of the first entries, written to
-    pages in any order: whole prompts, portions, single tokens, a position far out; part of a head rotated, all of it,
-    none; with and without the division; the half-apart pairing still what it was."""
+    """Division of every head by its root mean square and rotation of pairs of the first entries, (2i, 2i+1) or half the
+    rotated part apart, written to pages in any order: whole prompts, portions, single tokens, a position far out; part
+    of a head rotated, all of it, none; with and without the division; columns that start on a multiple of four (four
+    entries per lane, several heads per wave) and columns that do not (one entry per lane)."""
     from light_vllm_amd import mix_ops
+    from oracle import givozen_oracle
     g = torch.Generator().manual_seed(2)
     tol = 2e-5 if dtype == "float32" else 2e-2
-    for (H, G, D, Dv, dims, unit, page) in ((4, 2, 12, 10, 8, False, 16), (3, 1, 16, 8, 16, True, 16), (2, 2, 9, 5, 0, True, 8),
-                                            (1, 1, 40, 70, 2, False, 16), (6, 2, 32, 32, 32, False, 64)):
-        base, eps = 700.0, 1e-5
-        inv = mix_ops.rotary_inv_freq(max(dims, 2), base, device)
-        ld = H * D + G * D + G * Dv + 3
-        for lens, ctxs in (([21], [0]), ([2, 1, 5], [15, 70000, 3]), ([1], [16])):
-            B, T = len(lens), sum(lens)
-            proj = torch.randn(T, ld, generator=g).to(_dt(dtype))
-            need = [-(-(c + n) // page) for n, c in zip(lens, ctxs)]
-            perm = torch.randperm(sum(need) + 2, generator=g).tolist()
-            tables, at = [], 0
-            for nb in need:
-                tables.append(perm[at:at + nb])
-                at += nb
-            if max(need) > 64:      # the far position: only its own page matters
-                tables = [[perm[0]] * (nb - 1) + [perm[1 + b]] for b, nb in enumerate(need)]
-            kc = torch.zeros(sum(need) + 2, page, G, D, dtype=_dt(dtype), device=device)
-            vc = torch.zeros(sum(need) + 2, page, G, Dv, dtype=_dt(dtype), device=device)
-            step = K.make_step(lens, ctxs, list(range(B)), tables, device)
-            q = mix_ops.rotary_store(proj.to(device), 3, 3 + H * D, 3 + H * D + G * D, inv, None, kc, vc, step, H, G, D, Dv, dims,
-                                     interleaved=True, unit_eps=eps if unit else None).cpu().to(F64)
-            pf = proj.to(F64)
-            t0 = 0
-            for b, (n, c) in enumerate(zip(lens, ctxs)):
-                pos = list(range(c, c + n))
-                for hd in range(H + G):
-                    src = pf[t0:t0 + n, 3 + hd * D:3 + (hd + 1) * D]
-                    if unit:
-                        src = oracle.unit_rms(src, eps)
-                    want = oracle.rotate_pairs(src, pos, dims, base) if dims else src
-                    if hd < H:
-                        got = q[t0:t0 + n, hd * D:(hd + 1) * D]
-                    else:
-                        got = torch.stack([kc[tables[b][p // page], p % page, hd - H].cpu().to(F64) for p in pos])
-                    # an f32 angle at position 70000 is itself only good to half a hundredth
-                    lim = max(tol, 1e-2 if max(pos) > 60000 else 0.0) * max(1.0, want.abs().max().item())
-                    assert (got - want).abs().max().item() <= lim, (H, G, D, dims, unit, lens, hd)
-                gotv = torch.stack([vc[tables[b][p // page], p % page].cpu().to(F64).reshape(-1) for p in pos])
-                assert torch.equal(gotv, pf[t0:t0 + n, 3 + H * D + G * D:3 + H * D + G * D + G * Dv])
-                t0 += n
+    shapes = ((4, 2, 12, 10, 8, False, 16, True), (3, 1, 16, 8, 16, True, 16, True), (2, 2, 9, 5, 0, True, 8, True),
+              (1, 1, 40, 70, 2, False, 16, True), (6, 2, 32, 32, 32, False, 64, True), (2, 1, 128, 64, 64, True, 16, True),
+              (5, 5, 96, 32, 0, True, 16, True), (3, 1, 24, 8, 16, True, 16, False), (2, 2, 256, 16, 256, False, 16, True),
+              (7, 1, 8, 4, 8, True, 16, False))
+    for (H, G, D, Dv, dims, unit, page, inter) in shapes:
+        for pad in (3, 4):
+            base, eps = 700.0, 1e-5
+            inv = mix_ops.rotary_inv_freq(max(dims, 2), base, device)
+            ld = H * D + G * D + G * Dv + pad
+            for lens, ctxs in (([21], [0]), ([2, 1, 5], [15, 70000, 3]), ([1], [16])):
+                B, T = len(lens), sum(lens)
+                proj = torch.randn(T, ld, generator=g).to(_dt(dtype))
+                need = [-(-(c + n) // page) for n, c in zip(lens, ctxs)]
+                perm = torch.randperm(sum(min(nb, 8) for nb in need) + 2, generator=g).tolist()
+                tables, at = [], 0
+                for nb in need:       # a far position: only its own page matters
+                    tables.append([perm[at]] * (nb - min(nb, 8)) + perm[at:at + min(nb, 8)])
+                    at += min(nb, 8)
+                kc = torch.zeros(len(perm), page, G, D, dtype=_dt(dtype), device=device)
+                vc = torch.zeros(len(perm), page, G, Dv, dtype=_dt(dtype), device=device)
+                step = K.make_step(lens, ctxs, list(range(B)), tables, device)
+                q = mix_ops.rotary_store(proj.to(device), pad, pad + H * D, pad + H * D + G * D, inv, None, kc, vc, step, H, G, D, Dv, dims,
+                                         interleaved=inter, unit_eps=eps if unit else None).cpu().to(F64)
+                pf = proj.to(F64)
+                t0 = 0
+                for b, (n, c) in enumerate(zip(lens, ctxs)):
+                    pos = list(range(c, c + n))
+                    for hd in range(H + G):
+                        src = pf[t0:t0 + n, pad + hd * D:pad + (hd + 1) * D]
+                        if unit:
+                            src = oracle.unit_rms(src, eps)
+                        if dims and inter:
+                            want = oracle.rotate_pairs(src, pos, dims, base)
+                        elif dims:
+                            want = givozen_oracle.rotate(src, pos, [base ** (-2.0 * i / dims) for i in range(dims // 2)])
+                        else:
+                            want = src
+                        if hd < H:
+                            got = q[t0:t0 + n, hd * D:(hd + 1) * D]
+                        else:
+                            got = torch.stack([kc[tables[b][p // page], p % page, hd - H].cpu().to(F64) for p in pos])
+                        # an f32 angle at position 70000 is itself only good to half a hundredth
+                        lim = max(tol, 1e-2 if max(pos) > 60000 else 0.0) * max(1.0, want.abs().max().item())
+                        assert (got - want).abs().max().item() <= lim, (H, G, D, dims, unit, inter, pad, lens, hd)
+                    gotv = torch.stack([vc[tables[b][p // page], p % page].cpu().to(F64).reshape(-1) for p in pos])
+                    assert torch.equal(gotv, pf[t0:t0 + n, pad + H * D + G * D:pad + H * D + G * D + G * Dv])
+                    t0 += n
 
 
 def _paged(k, v, page, dtype, device, g):
