@@ -272,22 +272,41 @@ __global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) 
   for (int r = 0; r < DR; ++r)
     s[r] = (carry && live && row0 + r < p.D) ? sbase[static_cast<int64_t>(row0 + r) * p.Dv + col] : 0.0f;
   const T* proj = static_cast<const T*>(p.proj);
+  // A chunk's inputs are fetched into registers one chunk ahead (all of a thread's loads in flight together, while the
+  // chunk before is computed); silu is applied where they move on to LDS.
+  constexpr int NKQ = kLightChunk * DP / 256, NV = kLightChunk * kWave / 256;
+  float kreg[NKQ], qreg[NKQ], vreg[NV];
+  auto fetch = [&](int c0) {
+    const int cn = min(kLightChunk, n - c0);
+#pragma unroll
+    for (int it = 0; it < NKQ; ++it) {
+      const int x = threadIdx.x + it * 256;
+      const int tok = x / DP, d = x - tok * DP;
+      const T* row = proj + (static_cast<int64_t>(q0) + c0 + tok) * p.ld + h * p.D + d;
+      const bool in = tok < cn && d < p.D;
+      kreg[it] = in ? ldf(row + p.off_k) : 0.0f;
+      qreg[it] = in ? ldf(row + p.off_q) : 0.0f;
+    }
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int x = threadIdx.x + it * 256;
+      const int tok = x / kWave, cc = blockIdx.x * kWave + (x % kWave);
+      vreg[it] = (tok < cn && cc < p.Dv) ? ldf(proj + (static_cast<int64_t>(q0) + c0 + tok) * p.ld + p.off_v + h * p.Dv + cc) : 0.0f;
+    }
+  };
+  fetch(0);
   for (int c0 = 0; c0 < n; c0 += kLightChunk) {
     const int cn = min(kLightChunk, n - c0);
-    __syncthreads();                               // the previous chunk's shares have been added up
-    for (int x = threadIdx.x; x < cn * DP; x += blockDim.x) {
-      const int tok = x / DP, d = x - tok * DP;
-      const T* row = proj + (static_cast<int64_t>(q0) + c0 + tok) * p.ld;
-      const bool in = d < p.D;
-      k_lds[x] = in ? siluf_(ldf(row + p.off_k + h * p.D + d)) : 0.0f;
-      q_lds[x] = in ? siluf_(ldf(row + p.off_q + h * p.D + d)) : 0.0f;
+    // every wave is past the previous chunk's token loop: behind the barrier that followed it
+#pragma unroll
+    for (int it = 0; it < NKQ; ++it) {
+      k_lds[threadIdx.x + it * 256] = siluf_(kreg[it]);
+      q_lds[threadIdx.x + it * 256] = siluf_(qreg[it]);
     }
-    for (int x = threadIdx.x; x < cn * kWave; x += blockDim.x) {
-      const int tok = x / kWave, cc = blockIdx.x * kWave + (x % kWave);
-      const T* row = proj + (static_cast<int64_t>(q0) + c0 + tok) * p.ld;
-      v_lds[x] = cc < p.Dv ? siluf_(ldf(row + p.off_v + h * p.Dv + cc)) : 0.0f;
-    }
+#pragma unroll
+    for (int it = 0; it < NV; ++it) v_lds[threadIdx.x + it * 256] = siluf_(vreg[it]);
     __syncthreads();
+    if (c0 + kLightChunk < n) fetch(c0 + kLightChunk);
     for (int i = 0; i < cn; ++i) {
       const float vv = v_lds[i * kWave + lane];
       float po4[4] = {0.0f, 0.0f, 0.0f, 0.0f};     // four chains: one sum would be bound by its own latency

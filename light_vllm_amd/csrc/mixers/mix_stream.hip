@@ -484,6 +484,35 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   }
 }
 
+// The same for heads of many entries (a norm over a whole row of heads is one such head): one workgroup per (token, head),
+// four entries per thread and access.
+template <typename T>
+__global__ __launch_bounds__(256) void wide_head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate,
+                                                                  int64_t ld_gate, const float* __restrict__ norm_w,
+                                                                  T* __restrict__ out, int H, int Dv, float eps, int gate_act) {
+  __shared__ float red[4];
+  const int64_t item = blockIdx.x;
+  const int64_t t = item / H;
+  const int h = static_cast<int>(item - t * H);
+  const float* row = o + item * Dv;
+  float ss = 0.0f;
+  for (int e = threadIdx.x * 4; e < Dv; e += blockDim.x * 4) {
+    const float4 v = ld4(row + e);
+    ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+  }
+  ss = wave_sum(ss);
+  if (threadIdx.x % kWave == 0) red[threadIdx.x / kWave] = ss;
+  __syncthreads();
+  const float inv = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / static_cast<float>(Dv) + eps);
+  const T* grow = gate + t * ld_gate + static_cast<int64_t>(h) * Dv;
+  auto act = [&](float g) { return gate_act == LV_MIX_GATE_SILU ? siluf_(g) : sigmoidf_(g); };
+  for (int e = threadIdx.x * 4; e < Dv; e += blockDim.x * 4) {
+    const float4 v = ld4(row + e), w = ld4(norm_w + e), g = ld4(grow + e);
+    st4(out + item * Dv + e, float4{v.x * inv * w.x * act(g.x), v.y * inv * w.y * act(g.y), v.z * inv * w.z * act(g.z),
+                                    v.w * inv * w.w * act(g.w)});
+  }
+}
+
 }  // namespace lvmix
 
 using namespace lvmix;
@@ -627,6 +656,20 @@ int lv_head_norm_gate(const void* o, const void* gate, int64_t ld_gate, const vo
       (gate_act != LV_MIX_GATE_SILU && gate_act != LV_MIX_GATE_SIGMOID))
     return fail(-1, "lv_head_norm_gate: bad arguments");
   const int64_t items = T * H;
+  auto aligned = [](const void* q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+  if (Dv >= 512 && Dv % 4 == 0 && ld_gate % 4 == 0 && aligned(o) && aligned(gate) && aligned(norm_w) && aligned(out) &&
+      (dtype == LV_MIX_BF16 || dtype == LV_MIX_F32)) {
+    dim3 wgrid(static_cast<unsigned>(items)), wblock(256);
+    if (dtype == LV_MIX_BF16)
+      wide_head_norm_gate_kernel<bf16_t><<<wgrid, wblock, 0, as_stream(stream)>>>(
+          static_cast<const float*>(o), static_cast<const bf16_t*>(gate), ld_gate, static_cast<const float*>(norm_w),
+          static_cast<bf16_t*>(out), H, Dv, eps, gate_act);
+    else
+      wide_head_norm_gate_kernel<float><<<wgrid, wblock, 0, as_stream(stream)>>>(
+          static_cast<const float*>(o), static_cast<const float*>(gate), ld_gate, static_cast<const float*>(norm_w),
+          static_cast<float*>(out), H, Dv, eps, gate_act);
+    return launched("lv_head_norm_gate");
+  }
   dim3 grid(static_cast<unsigned>((items + 3) / 4)), block(256);
   if (dtype == LV_MIX_BF16)
     head_norm_gate_kernel<bf16_t><<<grid, block, 0, as_stream(stream)>>>(
