@@ -244,19 +244,28 @@ struct LightningParams {
 };
 
 
-// DR = rows of the state each of the four waves owns (4 * DR >= D; rows beyond D stay zero); lane = value column.
-// Tokens come in chunks of kLightChunk (fewer for large heads, whose staged rows are longer): silu of the chunk's queries, keys and values is staged in LDS by all threads
-// at once, every wave then walks the chunk alone (its rows of S need nobody else's), leaving its share of each
-// read-out in LDS; the four shares are added when the chunk is done.
-template <typename T, int DR>
-__global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) {
+// NW waves a workgroup, DR = rows of the state each wave owns (NW * DR >= D; rows beyond D stay zero); lane = value column.
+// Tokens come in chunks: the chunk's queries, keys and values are fetched into registers one chunk ahead and staged in LDS
+// with silu applied; every wave then walks the chunk alone (its rows of S need nobody else's) and leaves its share of each
+// read-out in LDS; the NW shares are added when the chunk is done. The token loop is a chain of LDS reads and multiply-adds
+// that only other waves on the SIMD can overlap, so a launch with few workgroups (few sequences or heads) splits the rows
+// over eight waves instead of four.
+template <int DR, int NW>
+struct LightningShape {
+  static constexpr int kDP = NW * DR;
+  static constexpr int kChunk = (kDP >= 128 || NW > 4) ? 16 : 32;     // what fits 64 KB of LDS with the shares of NW waves
+  static constexpr size_t kLds = sizeof(float) * (2 * kChunk * kDP + kChunk * kWave + kChunk * NW * kWave);
+};
+
+template <typename T, int DR, int NW>
+__global__ __launch_bounds__(NW * 64) void lightning_attn_kernel(LightningParams p) {
   extern __shared__ __attribute__((aligned(16))) float ll[];
-  constexpr int DP = 4 * DR;
-  constexpr int kLightChunk = DR >= 32 ? 16 : 32;
+  constexpr int DP = NW * DR, NT = NW * kWave;
+  constexpr int kLightChunk = LightningShape<DR, NW>::kChunk;
   float* k_lds = ll;                               // [chunk][DP]
   float* q_lds = k_lds + kLightChunk * DP;         // [chunk][DP]
   float* v_lds = q_lds + kLightChunk * DP;         // [chunk][64]
-  float* part_o = v_lds + kLightChunk * kWave;     // [chunk][4][64]
+  float* part_o = v_lds + kLightChunk * kWave;     // [chunk][NW][64]
   const int lane = threadIdx.x % kWave, rp = threadIdx.x / kWave;
   const int col = blockIdx.x * kWave + lane;
   const int h = blockIdx.y, b = blockIdx.z;
@@ -272,15 +281,13 @@ __global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) 
   for (int r = 0; r < DR; ++r)
     s[r] = (carry && live && row0 + r < p.D) ? sbase[static_cast<int64_t>(row0 + r) * p.Dv + col] : 0.0f;
   const T* proj = static_cast<const T*>(p.proj);
-  // A chunk's inputs are fetched into registers one chunk ahead (all of a thread's loads in flight together, while the
-  // chunk before is computed); silu is applied where they move on to LDS.
-  constexpr int NKQ = kLightChunk * DP / 256, NV = kLightChunk * kWave / 256;
+  constexpr int NKQ = kLightChunk * DP / NT, NV = (kLightChunk * kWave + NT - 1) / NT;
   float kreg[NKQ], qreg[NKQ], vreg[NV];
   auto fetch = [&](int c0) {
     const int cn = min(kLightChunk, n - c0);
 #pragma unroll
     for (int it = 0; it < NKQ; ++it) {
-      const int x = threadIdx.x + it * 256;
+      const int x = threadIdx.x + it * NT;
       const int tok = x / DP, d = x - tok * DP;
       const T* row = proj + (static_cast<int64_t>(q0) + c0 + tok) * p.ld + h * p.D + d;
       const bool in = tok < cn && d < p.D;
@@ -289,7 +296,7 @@ __global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) 
     }
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
-      const int x = threadIdx.x + it * 256;
+      const int x = threadIdx.x + it * NT;
       const int tok = x / kWave, cc = blockIdx.x * kWave + (x % kWave);
       vreg[it] = (tok < cn && cc < p.Dv) ? ldf(proj + (static_cast<int64_t>(q0) + c0 + tok) * p.ld + p.off_v + h * p.Dv + cc) : 0.0f;
     }
@@ -300,11 +307,12 @@ __global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) 
     // every wave is past the previous chunk's token loop: behind the barrier that followed it
 #pragma unroll
     for (int it = 0; it < NKQ; ++it) {
-      k_lds[threadIdx.x + it * 256] = siluf_(kreg[it]);
-      q_lds[threadIdx.x + it * 256] = siluf_(qreg[it]);
+      k_lds[threadIdx.x + it * NT] = siluf_(kreg[it]);
+      q_lds[threadIdx.x + it * NT] = siluf_(qreg[it]);
     }
 #pragma unroll
-    for (int it = 0; it < NV; ++it) v_lds[threadIdx.x + it * 256] = siluf_(vreg[it]);
+    for (int it = 0; it < NV; ++it)
+      if (threadIdx.x + it * NT < kLightChunk * kWave) v_lds[threadIdx.x + it * NT] = siluf_(vreg[it]);
     __syncthreads();
     if (c0 + kLightChunk < n) fetch(c0 + kLightChunk);
     for (int i = 0; i < cn; ++i) {
@@ -323,14 +331,16 @@ __global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) 
         po4[2] += s[r + 2] * q4.z;
         po4[3] += s[r + 3] * q4.w;
       }
-      part_o[(i * 4 + rp) * kWave + lane] = (po4[0] + po4[1]) + (po4[2] + po4[3]);
+      part_o[(i * NW + rp) * kWave + lane] = (po4[0] + po4[1]) + (po4[2] + po4[3]);
     }
     __syncthreads();
-    for (int x = threadIdx.x; x < cn * kWave; x += blockDim.x) {
+    for (int x = threadIdx.x; x < cn * kWave; x += NT) {
       const int tok = x / kWave, ln = x % kWave, cc = blockIdx.x * kWave + ln;
-      const float* po = part_o + tok * 4 * kWave + ln;
-      if (cc < p.Dv)
-        p.o[((static_cast<int64_t>(q0) + c0 + tok) * p.H + h) * p.Dv + cc] = (po[0] + po[kWave]) + (po[2 * kWave] + po[3 * kWave]);
+      const float* po = part_o + tok * NW * kWave + ln;
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NW; w += 2) sum += po[w * kWave] + po[(w + 1) * kWave];
+      if (cc < p.Dv) p.o[((static_cast<int64_t>(q0) + c0 + tok) * p.H + h) * p.Dv + cc] = sum;
     }
   }
   if (live) {
@@ -340,19 +350,26 @@ __global__ __launch_bounds__(256) void lightning_attn_kernel(LightningParams p) 
   }
 }
 
-template <typename T, int DR>
+template <typename T, int DR, int NW>
 static void lightning_launch(const LightningParams& p, dim3 grid, hipStream_t s) {
-  constexpr int chunk = DR >= 32 ? 16 : 32;
-  const size_t shm = sizeof(float) * (2 * chunk * 4 * DR + chunk * kWave + chunk * 4 * kWave);
-  lightning_attn_kernel<T, DR><<<grid, dim3(256), shm, s>>>(p);
+  lightning_attn_kernel<T, DR, NW><<<grid, dim3(NW * kWave), LightningShape<DR, NW>::kLds, s>>>(p);
 }
 
 template <typename T>
-static int lightning_dispatch(const LightningParams& p, dim3 grid, hipStream_t s) {
-  if (p.D <= 32) lightning_launch<T, 8>(p, grid, s);
-  else if (p.D <= 64) lightning_launch<T, 16>(p, grid, s);
-  else if (p.D <= 128) lightning_launch<T, 32>(p, grid, s);
-  else lightning_launch<T, 64>(p, grid, s);
+static int lightning_dispatch(const LightningParams& p, int B, hipStream_t s) {
+  dim3 grid((p.Dv + kWave - 1) / kWave, p.H, B);
+  // fewer than four workgroups a compute unit: eight waves each, so that a SIMD still holds four
+  const bool eight = static_cast<int64_t>(grid.x) * grid.y * grid.z < 4 * 256 && p.D > 16 && p.D <= 128;
+  if (eight) {
+    if (p.D <= 32) lightning_launch<T, 4, 8>(p, grid, s);
+    else if (p.D <= 64) lightning_launch<T, 8, 8>(p, grid, s);
+    else lightning_launch<T, 16, 8>(p, grid, s);
+  } else {
+    if (p.D <= 32) lightning_launch<T, 8, 4>(p, grid, s);
+    else if (p.D <= 64) lightning_launch<T, 16, 4>(p, grid, s);
+    else if (p.D <= 128) lightning_launch<T, 32, 4>(p, grid, s);
+    else lightning_launch<T, 64, 4>(p, grid, s);
+  }
   return 0;
 }
 
@@ -480,9 +497,8 @@ int lv_lightning_attn(const void* proj, int64_t ld, int off_q, int off_k, int of
   if (D > 256) return fail(-2, "lv_lightning_attn: key size %d above 256", D);
   LightningParams p{proj, ld, off_q, off_k, off_v, static_cast<const float*>(decay), static_cast<float*>(state), cu_q, ctx_lens,
                     slots, static_cast<float*>(o), H, D, Dv};
-  dim3 grid((Dv + kWave - 1) / kWave, H, B);
-  if (dtype == LV_MIX_BF16) lightning_dispatch<bf16_t>(p, grid, as_stream(stream));
-  else if (dtype == LV_MIX_F32) lightning_dispatch<float>(p, grid, as_stream(stream));
+  if (dtype == LV_MIX_BF16) lightning_dispatch<bf16_t>(p, B, as_stream(stream));
+  else if (dtype == LV_MIX_F32) lightning_dispatch<float>(p, B, as_stream(stream));
   else return fail(-1, "lv_lightning_attn: dtype %d", dtype);
   return launched("lv_lightning_attn");
 }

@@ -190,12 +190,14 @@ def case_lightning(device, dtype):
     """The decaying state against the token-by-token recurrence: whole prompts, the same prompts in portions and single
     tokens through state slots in any order, a slot that held another sequence before, decays of 0 and 1 and near 1,
     key sizes that are no multiple of four, value sizes above one wave, rows of heads short and long (the norm over all
-    heads, with the gate behind it, has a form of its own for long rows)."""
+    heads, with the gate behind it, has a form of its own for long rows), launches of few workgroups and of many (the state's
+    rows are then split over eight waves or four)."""
     from light_vllm_amd import mix_ops
     g = torch.Generator().manual_seed(3)
     tol = 2e-5 if dtype == "float32" else 2e-2
     for (H, D, Dv, decay) in ((3, 8, 12, [0.5, 0.9, 0.995]), (1, 40, 70, [1.0]), (2, 6, 5, [0.0, 0.8]), (4, 16, 16, [0.6, 0.8, 0.95, 0.999]),
-                              (2, 128, 64, [0.99, 0.3]), (1, 130, 8, [0.9]), (4, 16, 160, [0.9, 0.5, 0.99, 0.7])):
+                              (2, 128, 64, [0.99, 0.3]), (1, 130, 8, [0.9]), (4, 16, 160, [0.9, 0.5, 0.99, 0.7]), (1, 100, 128, [0.95]), (2, 24, 40, [0.9, 0.8]),
+                              (128, 40, 512, [0.5 + 0.499 * i / 127 for i in range(128)]), (64, 100, 1024, [0.9] * 64)):
         Wd, eps = 24, 1e-5
         m = {"heads": H, "dim": D, "vdim": Dv, "decay": decay}
         shapes = {"q": (H * D, Wd), "k": (H * D, Wd), "v": (H * Dv, Wd), "g": (H * Dv, Wd), "o": (Wd, H * Dv), "norm": (H * Dv,)}
