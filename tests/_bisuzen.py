@@ -84,6 +84,22 @@ CFG_WIDE = {
     ],
 }
 
+# head sizes of a real model's order, windows, kept tokens and chunks longer than a 64-token page and a 64-key tile, prompts
+# of a few hundred tokens (tests/_bisuzen_cases.py::case_engine_long_windows)
+CFG_LONG = {
+    "architecture": "Bisuzen", "vocab": 211, "width": 96, "norm": {"eps": 1e-6}, "logit_scale": 1.25,
+    "loop": {"start": 0, "stop": 1, "times": 2},
+    "layers": [
+        {"type": "parallel",
+         "mixer": {"left": {"heads": 6, "kv_heads": 3, "dim": 64, "vdim": 32, "scale": 0.125, "mask": {"size": 70, "keep_first": 3},
+                            "rot": {"base": 20000.0, "dims": 32}},
+                   "right": {"heads": 2, "dim": 32, "vdim": 96, "decay": [0.97, 0.999]}},
+         "mlp": {"kind": "moe", "expert": {"ff": 64}, "router": {"experts": 10, "identity": 2, "top": 3, "groups": {"count": 3, "keep": 2}}}},
+        {"type": "attention", "mixer": {"heads": 4, "kv_heads": 1, "dim": 32, "vdim": 64, "scale": 0.2, "mask": {"size": 90}},
+         "mlp": {"kind": "dense", "ff": 160}},
+    ],
+}
+
 
 def random_config(seed: int) -> dict:
     """A configuration drawn from lists of sizes: layer count and kinds, loop, head counts and sizes, rotated part,

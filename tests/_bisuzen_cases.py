@@ -504,6 +504,26 @@ def case_engine_random_config(device, dtype, tmp_path, seed):
             assert err <= K.TOL[dtype], (seed, name, i, err, cfg)
 
 
+def case_engine_long_windows(device, dtype, tmp_path):
+    """Windows, kept tokens and chunks that span several pages and key tiles: a prompt of 330 tokens whole, cut into
+    portions at odd places beside the single tokens of another request, and decoded token by token across the edges."""
+    cfg = K.CFG_LONG
+    model_dir, weights = _model(tmp_path, cfg, 11)
+    prompts = {"a": K.tokens_for(cfg, 330, 41), "b": K.tokens_for(cfg, 100, 42)}
+    want, decided = _oracle_runs(cfg, weights, prompts, dtype)
+    schedules = {
+        "whole": [[("a", 330)], [("b", 100)]],
+        "mixed": [[("a", 67)], [("a", 2), ("b", 60)], [("a", 111), ("b", 1)], [("a", 1), ("b", 1)], [("a", 89), ("b", 1)]]
+                 + [[("a", 1), ("b", 1)]] * 37 + [[("a", 23)]],
+    }
+    for name, schedule in schedules.items():
+        got = K.replay(model_dir, dtype, device, prompts, schedule, max_tokens=512, page=64, slots=2)
+        for i, logits in got.items():
+            rows = [j for j in decided[i] if j < len(logits)]
+            err = K.rel_err(logits[rows], want[i][rows])
+            assert err <= K.TOL[dtype], (name, i, err)
+
+
 def case_engine_reuse(device, dtype, tmp_path):
     """More requests than state slots and more tokens than pages: both are given back and used again,
     in another order, and a sequence that starts on used pages and a used slot starts from nothing."""

@@ -49,6 +49,10 @@ def test_engine_random_configs(tmp_path, seed):
     C.case_engine_random_config(DEV, "float32", tmp_path, seed)
 
 
+def test_engine_long_windows(tmp_path):
+    C.case_engine_long_windows(DEV, "float32", tmp_path)
+
+
 def test_engine_reuse_of_pages_and_slots(tmp_path):
     C.case_engine_reuse(DEV, "float32", tmp_path)
 

@@ -61,6 +61,11 @@ def test_engine_random_configs(gpu, tmp_path, seed, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_engine_long_windows(gpu, tmp_path, dtype):
+    C.case_engine_long_windows(DEV, dtype, tmp_path)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_engine_reuse_of_pages_and_slots(gpu, tmp_path, dtype):
     C.case_engine_reuse(DEV, dtype, tmp_path)
 
